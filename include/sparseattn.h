@@ -1,0 +1,117 @@
+/*
+ * sparseattn.h - C ABI of the MI355X (gfx950) block-sparse attention forward library
+ * (libsparseattn_hip.so).
+ *
+ * The library replaces the two device kernels of tomatillos/sparseattention and nothing else:
+ *
+ *   sa_mask_classify          replaces the launch in compute_mask_kernel
+ *                             (sparseattention/mask_utils.py:85-107, kernel :47-82)
+ *   sa_sparse_attention_fwd   replaces the launch in sparse_attention
+ *                             (sparseattention/sparse_attn_kernel.py:149-185, kernels :10-63, :74-146)
+ *
+ * Conventions
+ *   - All pointers are DEVICE pointers owned by the caller.  The library allocates nothing,
+ *     frees nothing and keeps no pointer after a call returns.
+ *   - Strides are in ELEMENTS of the tensor they describe (bytes for the bool mask), exactly what
+ *     torch.Tensor.stride() returns, and may be 0 on broadcast dimensions.
+ *   - `stream` is a hipStream_t (NULL = the default stream).  Calls only enqueue work; they never
+ *     synchronise the host with the device.
+ *   - Return value: SA_OK or a negative SA_ERR_* code; sa_last_error() then gives a message
+ *     (thread-local).  Argument errors are detected on the host before any kernel is launched.
+ *   - Mask semantics: a byte != 0 means "this query may attend to this key" (torch bool masks).
+ *     A tile of BQ x BK entries is FULL when every entry is set, EMPTY when none is, otherwise
+ *     PARTIAL (mask_utils.py:34-40).
+ */
+#ifndef SPARSEATTN_H
+#define SPARSEATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SA_ABI_VERSION 1
+
+enum sa_status {
+    SA_OK = 0,
+    SA_ERR_INVALID_ARGUMENT = -1, /* null pointer, non-positive size, Sq % BQ != 0, Sk % BK != 0 ... */
+    SA_ERR_UNSUPPORTED = -2,      /* valid request the gfx950 kernels have no instantiation for */
+    SA_ERR_WORKSPACE = -3,        /* workspace missing or smaller than sa_mask_classify_workspace_bytes */
+    SA_ERR_HIP = -4               /* the HIP runtime refused the launch */
+};
+
+enum sa_dtype {
+    SA_DTYPE_BF16 = 0,
+    SA_DTYPE_FP16 = 1
+};
+
+/* ABI version of the loaded library (== SA_ABI_VERSION it was built with). */
+int sa_abi_version(void);
+
+/* Message for the last error returned on the calling thread ("" if none). */
+const char *sa_last_error(void);
+
+/*
+ * Bytes of device scratch sa_mask_classify needs for this problem: one class byte per tile of
+ * every DISTINCT mask plane (dimensions whose mask stride is 0 count once).  Returns 0 on
+ * invalid arguments.
+ */
+size_t sa_mask_classify_workspace_bytes(const int64_t mask_strides[4], int B, int H, int Sq, int Sk, int BQ,
+                                        int BK);
+
+/*
+ * Tile classification.  Replaces compute_mask_kernel's launch (mask_utils.py:96-106).
+ *
+ *   mask        bool [B,H,Sq,Sk] addressed through mask_strides (any strides, 0 allowed).
+ *   full_ids    int32 [B,H,Sq/BQ,Sk/BK]: ascending KV-tile indices of FULL tiles ("unmasked_kv_ids");
+ *   full_lens   int32 [B,H,Sq/BQ]: how many of them are valid ("unmasked_lens");
+ *   part_ids / part_lens: the same for PARTIAL tiles ("masked_kv_ids", "masked_lens").
+ *               Slots at positions >= the count are left untouched, as in the reference, which
+ *               allocates them with torch.empty (mask_utils.py:91-94).
+ *   Output strides may be 0 on b and/or h when the mask's stride is 0 there (the result is the
+ *   same for every plane; it is then computed and written once).
+ *   workspace   device scratch of at least sa_mask_classify_workspace_bytes(...) bytes; contents
+ *               need not be initialised and are garbage afterwards.
+ *
+ * Any BQ, BK with Sq % BQ == 0 and Sk % BK == 0 is accepted.  Masks whose last dimension is
+ * contiguous and 16-byte aligned with 16 <= BK <= 1024, BK a power of two, take the wide-load
+ * kernel; everything else takes a slower generic kernel with identical results.
+ */
+int sa_mask_classify(const uint8_t *mask, const int64_t mask_strides[4], int B, int H, int Sq, int Sk, int BQ,
+                     int BK, int32_t *full_ids, const int64_t full_ids_strides[4], int32_t *full_lens,
+                     const int64_t full_lens_strides[3], int32_t *part_ids, const int64_t part_ids_strides[4],
+                     int32_t *part_lens, const int64_t part_lens_strides[3], void *workspace,
+                     size_t workspace_bytes, void *stream);
+
+/*
+ * Block-sparse flash-attention forward.  Replaces sparse_attention_kernel's launch
+ * (sparse_attn_kernel.py:167-184).
+ *
+ *   q,o  [B,H,Sq,D]; k,v [B,H,Sk,D]; dtype selects bf16 or fp16 for all four.  The last
+ *   dimension must be contiguous (stride 1), every other stride a multiple of 8 elements and
+ *   the base pointers 16-byte aligned; otherwise SA_ERR_UNSUPPORTED (copy to a contiguous tensor).
+ *   mask and the four metadata tensors are as in sa_mask_classify; only ids[..., :len] are read.
+ *   sm_scale_log2 = softmax scale divided by ln 2 (the reference uses D^-0.5 / ln 2,
+ *   sparse_attn_kernel.py:152); scores are exponentiated with exp2.
+ *
+ * For each query tile: FULL tiles first without reading the mask, then PARTIAL tiles with the
+ * mask applied, online softmax state in fp32, P rounded to the input dtype before P.V
+ * (sparse_attn_kernel.py:61).  Rows with no attended key produce 0 (the reference produces NaN).
+ *
+ * Supported: D in {64,128}; BQ in {32,64,128}; BK a power of two >= 16.
+ */
+int sa_sparse_attention_fwd(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                            const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
+                            const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
+                            const int64_t full_ids_strides[4], const int32_t *full_lens,
+                            const int64_t full_lens_strides[3], const int32_t *part_ids,
+                            const int64_t part_ids_strides[4], const int32_t *part_lens,
+                            const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int D, int BQ, int BK,
+                            int dtype, float sm_scale_log2, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPARSEATTN_H */

@@ -1,0 +1,189 @@
+"""CPU oracle for the block-sparse attention forward path.  TEST INFRASTRUCTURE ONLY.
+
+Only tests, the smoke check and the benchmark's CPU-baseline leg may import this package.
+The product (``sparseattention_amd``) never does: it fails loudly when its HIP library is
+missing instead of falling back to anything in here.
+
+Two restatements of the reference algorithm live here:
+
+* ``sparse_oracle.c`` (built into ``liboracle.so`` by ``oracle/Makefile``), wrapped by
+  :func:`classify` and :func:`forward`;
+* the numpy functions :func:`classify_numpy` and :func:`forward_dense_fp64`, written a
+  different way (per-tile popcount by reshape; dense fp64 softmax) so that the two can be
+  checked against each other and against closed forms.
+
+Reference lines followed: ``sparseattention/mask_utils.py:14-44`` (classification) and
+``sparseattention/sparse_attn_kernel.py:28-63, 103-146, 152`` (two-pass forward).
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+import os
+import subprocess
+from dataclasses import dataclass
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    """Compile ``sparse_oracle.c`` with gcc (the recipe is ``oracle/Makefile``)."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.run(["make", "-C", _HERE, "liboracle.so"], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+def _load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        build()
+    lib = ctypes.CDLL(_LIB_PATH)
+    i32p = ctypes.POINTER(ctypes.c_int32)
+    i64p = ctypes.POINTER(ctypes.c_int64)
+    f32p = ctypes.POINTER(ctypes.c_float)
+    u8p = ctypes.POINTER(ctypes.c_uint8)
+    lib.oracle_classify.restype = ctypes.c_int
+    lib.oracle_classify.argtypes = [u8p, i64p] + [ctypes.c_int] * 6 + [i32p] * 4
+    lib.oracle_forward.restype = ctypes.c_int
+    lib.oracle_forward.argtypes = (
+        [f32p, f32p, f32p, f32p, u8p, i64p, i32p, i32p, i32p, i32p] + [ctypes.c_int] * 7 + [ctypes.c_float, ctypes.c_int]
+    )
+    lib.oracle_max_threads.restype = ctypes.c_int
+    _lib = lib
+    return lib
+
+
+def max_threads() -> int:
+    """Threads the C oracle's OpenMP loops will use."""
+    return int(_load().oracle_max_threads())
+
+
+@dataclass
+class OracleMetadata:
+    """Same four fields, same order, as ``MaskMetadata`` (mask_utils.py:6-11), as numpy int32 arrays."""
+
+    unmasked_kv_ids: np.ndarray
+    unmasked_lens: np.ndarray
+    masked_kv_ids: np.ndarray
+    masked_lens: np.ndarray
+
+
+def _ptr(a: np.ndarray, ty):
+    return a.ctypes.data_as(ctypes.POINTER(ty))
+
+
+def _mask_view(mask: np.ndarray):
+    """Return (uint8 view, strides-in-bytes as int64[4]) for a 4-d bool/uint8 array of any strides."""
+    if mask.ndim != 4:
+        raise ValueError("mask must be 4-d [B,H,Sq,Sk] (broadcast views are fine)")
+    if mask.dtype == np.bool_:
+        mask = mask.view(np.uint8)
+    if mask.dtype != np.uint8:
+        raise ValueError("mask must be bool")
+    strides = np.array(mask.strides, dtype=np.int64)
+    return mask, strides
+
+
+def classify(mask: np.ndarray, BQ: int, BK: int) -> OracleMetadata:
+    """C restatement of ``compute_mask_slow`` (mask_utils.py:14-44).  Tail slots are -1."""
+    lib = _load()
+    B, H, Sq, Sk = mask.shape
+    if Sq % BQ or Sk % BK:
+        raise ValueError("Sq % BLOCK_Q and Sk % BLOCK_K must be 0")
+    m8, strides = _mask_view(mask)
+    nQ, nK = Sq // BQ, Sk // BK
+    fid = np.empty((B, H, nQ, nK), np.int32)
+    pid = np.empty((B, H, nQ, nK), np.int32)
+    fl = np.empty((B, H, nQ), np.int32)
+    pl = np.empty((B, H, nQ), np.int32)
+    rc = lib.oracle_classify(
+        _ptr(m8, ctypes.c_uint8), _ptr(strides, ctypes.c_int64), B, H, Sq, Sk, BQ, BK,
+        _ptr(fid, ctypes.c_int32), _ptr(fl, ctypes.c_int32), _ptr(pid, ctypes.c_int32), _ptr(pl, ctypes.c_int32),
+    )
+    if rc != 0:
+        raise RuntimeError(f"oracle_classify failed: {rc}")
+    return OracleMetadata(fid, fl, pid, pl)
+
+
+def classify_numpy(mask: np.ndarray, BQ: int, BK: int) -> OracleMetadata:
+    """Vectorised popcount classification; independent of the C loop.  Tail slots are -1."""
+    B, H, Sq, Sk = mask.shape
+    nQ, nK = Sq // BQ, Sk // BK
+    m = np.ascontiguousarray(np.broadcast_to(mask, (B, H, Sq, Sk))).astype(bool)
+    counts = m.reshape(B, H, nQ, BQ, nK, BK).sum(axis=(3, 5), dtype=np.int64)
+    full = counts == BQ * BK
+    part = (counts > 0) & ~full
+
+    def compact(flags):
+        lens = flags.sum(-1).astype(np.int32)
+        # stable sort puts flagged tile indices first, ascending
+        order = np.argsort(~flags, axis=-1, kind="stable").astype(np.int32)
+        pos = np.arange(nK, dtype=np.int32)
+        ids = np.where(pos < lens[..., None], order, np.int32(-1)).astype(np.int32)
+        return ids, lens
+
+    fid, fl = compact(full)
+    pid, pl = compact(part)
+    return OracleMetadata(fid, fl, pid, pl)
+
+
+def forward(q, k, v, mask, BQ: int, BK: int, meta: OracleMetadata | None = None, p_round: int = 0) -> np.ndarray:
+    """C restatement of the two-pass forward (sparse_attn_kernel.py:28-63, 103-146).
+
+    ``q, k, v``: float32 arrays [B,H,S,D] (widen bf16/fp16 inputs exactly before calling).
+    ``p_round``: 0 keep P in fp32, 1 round P to bf16 before P·V, 2 round to fp16.
+    Returns float32 [B,H,Sq,D].
+    """
+    lib = _load()
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    k = np.ascontiguousarray(k, dtype=np.float32)
+    v = np.ascontiguousarray(v, dtype=np.float32)
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    mask = np.broadcast_to(mask, (B, H, Sq, Sk))
+    if meta is None:
+        meta = classify(mask, BQ, BK)
+    m8, strides = _mask_view(mask)
+    out = np.empty_like(q)
+    scale_log2 = D ** -0.5 / math.log(2.0)
+    ids_f = np.ascontiguousarray(meta.unmasked_kv_ids, dtype=np.int32)
+    len_f = np.ascontiguousarray(meta.unmasked_lens, dtype=np.int32)
+    ids_p = np.ascontiguousarray(meta.masked_kv_ids, dtype=np.int32)
+    len_p = np.ascontiguousarray(meta.masked_lens, dtype=np.int32)
+    rc = lib.oracle_forward(
+        _ptr(q, ctypes.c_float), _ptr(k, ctypes.c_float), _ptr(v, ctypes.c_float), _ptr(out, ctypes.c_float),
+        _ptr(m8, ctypes.c_uint8), _ptr(strides, ctypes.c_int64),
+        _ptr(ids_f, ctypes.c_int32), _ptr(len_f, ctypes.c_int32), _ptr(ids_p, ctypes.c_int32), _ptr(len_p, ctypes.c_int32),
+        B, H, Sq, Sk, D, BQ, BK, ctypes.c_float(scale_log2), p_round,
+    )
+    if rc != 0:
+        raise RuntimeError(f"oracle_forward failed: {rc}")
+    return out
+
+
+def forward_dense_fp64(q, k, v, mask) -> np.ndarray:
+    """Dense masked softmax attention in float64: softmax(QK^T/sqrt(D) + (mask ? 0 : -inf)) V.
+
+    Rows with no attended key give 0.  Quadratic memory: small shapes only.
+    """
+    q = np.asarray(q, dtype=np.float64)
+    k = np.asarray(k, dtype=np.float64)
+    v = np.asarray(v, dtype=np.float64)
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    mask = np.broadcast_to(np.asarray(mask).astype(bool), (B, H, Sq, Sk))
+    s = np.einsum("bhqd,bhkd->bhqk", q, k) / math.sqrt(D)
+    s = np.where(mask, s, -np.inf)
+    mx = s.max(axis=-1, keepdims=True)
+    mx = np.where(np.isfinite(mx), mx, 0.0)
+    p = np.exp(s - mx)
+    den = p.sum(axis=-1, keepdims=True)
+    p = np.divide(p, den, out=np.zeros_like(p), where=den > 0)
+    return np.einsum("bhqk,bhkd->bhqd", p, v)

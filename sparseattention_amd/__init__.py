@@ -1,0 +1,15 @@
+"""MI355X-native block-sparse attention forward.
+
+Same Python surface as tomatillos/sparseattention for its one hot path:
+
+* :func:`sparse_attention` (reference: ``sparseattention/sparse_attn_kernel.py:149``)
+* :func:`compute_mask_kernel`, :func:`compute_mask_slow`, :class:`MaskMetadata`
+  (reference: ``sparseattention/mask_utils.py:85``, ``:14``, ``:6``)
+
+The device work is done by hand-written gfx950 HIP kernels in ``libsparseattn_hip.so``
+behind the C ABI of ``include/sparseattn.h``.
+"""
+from .mask_utils import MaskMetadata, compute_mask_kernel, compute_mask_slow
+from .sparse_attn_kernel import sparse_attention
+
+__all__ = ["MaskMetadata", "compute_mask_kernel", "compute_mask_slow", "sparse_attention"]

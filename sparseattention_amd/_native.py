@@ -1,0 +1,88 @@
+"""ctypes binding of libsparseattn_hip.so (the C ABI declared in include/sparseattn.h).
+
+There is no fallback: if the library is missing or a call fails, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libsparseattn_hip.so")
+
+SA_ABI_VERSION = 1
+SA_OK = 0
+SA_ERR_INVALID_ARGUMENT = -1
+SA_ERR_UNSUPPORTED = -2
+SA_ERR_WORKSPACE = -3
+SA_ERR_HIP = -4
+
+SA_DTYPE_BF16 = 0
+SA_DTYPE_FP16 = 1
+
+#: every symbol include/sparseattn.h declares
+EXPORTS = (
+    "sa_abi_version",
+    "sa_last_error",
+    "sa_mask_classify_workspace_bytes",
+    "sa_mask_classify",
+    "sa_sparse_attention_fwd",
+)
+
+_lib = None
+
+_i64p = ctypes.POINTER(ctypes.c_int64)
+_vp = ctypes.c_void_p
+
+
+class SparseAttnError(RuntimeError):
+    """A call into libsparseattn_hip.so returned an error code."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"libsparseattn_hip error {code}: {message}")
+        self.code = code
+
+
+def load() -> ctypes.CDLL:
+    """Load the in-tree HIP library.  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m sparseattention_amd.build` "
+            "(hipcc, gfx950).  There is no CPU or PyTorch fallback for the attention path."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.sa_abi_version.restype = ctypes.c_int
+    lib.sa_abi_version.argtypes = []
+    lib.sa_last_error.restype = ctypes.c_char_p
+    lib.sa_last_error.argtypes = []
+    lib.sa_mask_classify_workspace_bytes.restype = ctypes.c_size_t
+    lib.sa_mask_classify_workspace_bytes.argtypes = [_i64p] + [ctypes.c_int] * 6
+    lib.sa_mask_classify.restype = ctypes.c_int
+    lib.sa_mask_classify.argtypes = (
+        [_vp, _i64p] + [ctypes.c_int] * 6 + [_vp, _i64p] * 4 + [_vp, ctypes.c_size_t, _vp]
+    )
+    lib.sa_sparse_attention_fwd.restype = ctypes.c_int
+    lib.sa_sparse_attention_fwd.argtypes = (
+        [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [ctypes.c_int] * 8 + [ctypes.c_float, _vp]
+    )
+    if lib.sa_abi_version() != SA_ABI_VERSION:
+        raise RuntimeError(f"libsparseattn_hip ABI {lib.sa_abi_version()} != expected {SA_ABI_VERSION}")
+    _lib = lib
+    return lib
+
+
+def strides(values):
+    """int64[n] ctypes array from an iterable of strides."""
+    values = tuple(int(v) for v in values)
+    return (ctypes.c_int64 * len(values))(*values)
+
+
+def check(rc: int) -> None:
+    if rc != SA_OK:
+        msg = load().sa_last_error().decode("utf-8", "replace")
+        if rc == SA_ERR_INVALID_ARGUMENT:
+            raise ValueError(f"libsparseattn_hip: {msg}")
+        raise SparseAttnError(rc, msg)

@@ -1,0 +1,49 @@
+// Internal declarations shared by the C-ABI translation unit and the kernel translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sa {
+
+// ---- mask classification -------------------------------------------------------------------------
+struct ClassifyParams {
+    const uint8_t *mask;
+    int64_t sb, sh, sq, sk;  // mask strides in bytes over the DISTINCT planes (sb/sh unused when uB/uH == 1)
+    uint8_t *cls;            // [uB*uH, nQ, nK] class bytes: 0 empty, 1 partial, 2 full
+    int uB, uH;              // distinct planes along b and h
+    int Sq, Sk, BQ, BK, nQ, nK;
+    int lbk;                 // log2(BK) (wide kernel only)
+};
+
+struct CompactParams {
+    const uint8_t *cls;
+    int uH;                // distinct planes along h in cls
+    int bcast_b, bcast_h;  // 1: every output plane along that dimension reads class plane 0
+    int oB, oH;            // output planes to write
+    int nQ, nK;
+    int32_t *full_ids, *full_lens, *part_ids, *part_lens;
+    int64_t fis[4], fls[3], pis[4], pls[3];  // output strides in elements
+};
+
+hipError_t launch_classify(const ClassifyParams &p, bool wide, hipStream_t stream);
+hipError_t launch_compact(const CompactParams &p, hipStream_t stream);
+
+// ---- block-sparse forward ------------------------------------------------------------------------
+struct FwdParams {
+    const uint16_t *q, *k, *v;
+    uint16_t *o;
+    const uint8_t *mask;
+    const int32_t *full_ids, *full_lens, *part_ids, *part_lens;
+    int64_t qs[3], ks[3], vs[3], os[3];  // b, h, s strides in elements (d stride is 1)
+    int64_t ms[4];                        // mask strides in bytes
+    int64_t fis[4], fls[3], pis[4], pls[3];
+    int B, H, Sq, Sk, nQ;
+    int BK, lbk;    // KV tile width and its log2
+    int mask_vec4;  // 1: mask columns are contiguous and 4-byte aligned, so 4 entries load as one dword
+    float scale;    // softmax scale / ln 2
+};
+
+// dtype: 0 bf16, 1 fp16.  Returns hipErrorInvalidValue when no instantiation matches (D, BQ).
+hipError_t launch_fwd(const FwdParams &p, int dtype, int D, int BQ, hipStream_t stream);
+
+}  // namespace sa

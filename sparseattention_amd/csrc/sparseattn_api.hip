@@ -1,0 +1,215 @@
+// C ABI of libsparseattn_hip.so: argument validation, broadcast-plane folding and kernel dispatch.
+// The declarations and their contracts live in include/sparseattn.h.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "kernels.h"
+#include "sparseattn.h"
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int log2_exact(int x) {  // -1 unless x is a power of two
+    if (x <= 0 || (x & (x - 1))) return -1;
+    int l = 0;
+    while ((1 << l) < x) l++;
+    return l;
+}
+
+bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+// Shape checks shared by both entry points.  Returns SA_OK or an error code (message set).
+int check_tiling(int B, int H, int Sq, int Sk, int BQ, int BK) {
+    if (B <= 0 || H <= 0 || Sq <= 0 || Sk <= 0) return fail(SA_ERR_INVALID_ARGUMENT, "B, H, Sq, Sk must be positive (got %d, %d, %d, %d)", B, H, Sq, Sk);
+    if (BQ <= 0 || BK <= 0) return fail(SA_ERR_INVALID_ARGUMENT, "BLOCK_Q and BLOCK_K must be positive (got %d, %d)", BQ, BK);
+    if (Sq % BQ) return fail(SA_ERR_INVALID_ARGUMENT, "Sq (%d) must be a multiple of BLOCK_Q (%d)", Sq, BQ);
+    if (Sk % BK) return fail(SA_ERR_INVALID_ARGUMENT, "Sk (%d) must be a multiple of BLOCK_K (%d)", Sk, BK);
+    return SA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int sa_abi_version(void) { return SA_ABI_VERSION; }
+
+const char *sa_last_error(void) { return g_error; }
+
+size_t sa_mask_classify_workspace_bytes(const int64_t mask_strides[4], int B, int H, int Sq, int Sk, int BQ, int BK) {
+    if (!mask_strides || check_tiling(B, H, Sq, Sk, BQ, BK) != SA_OK) return 0;
+    const size_t uB = (mask_strides[0] == 0) ? 1 : (size_t)B;
+    const size_t uH = (mask_strides[1] == 0) ? 1 : (size_t)H;
+    return uB * uH * (size_t)(Sq / BQ) * (size_t)(Sk / BK);
+}
+
+int sa_mask_classify(const uint8_t *mask, const int64_t mask_strides[4], int B, int H, int Sq, int Sk, int BQ, int BK,
+                     int32_t *full_ids, const int64_t full_ids_strides[4], int32_t *full_lens,
+                     const int64_t full_lens_strides[3], int32_t *part_ids, const int64_t part_ids_strides[4],
+                     int32_t *part_lens, const int64_t part_lens_strides[3], void *workspace, size_t workspace_bytes,
+                     void *stream) {
+    g_error[0] = 0;
+    if (!mask || !mask_strides || !full_ids || !full_ids_strides || !full_lens || !full_lens_strides || !part_ids ||
+        !part_ids_strides || !part_lens || !part_lens_strides)
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_classify: null pointer argument");
+    if (const int rc = check_tiling(B, H, Sq, Sk, BQ, BK)) return rc;
+    const size_t need = sa_mask_classify_workspace_bytes(mask_strides, B, H, Sq, Sk, BQ, BK);
+    if (!workspace || workspace_bytes < need)
+        return fail(SA_ERR_WORKSPACE, "sa_mask_classify: workspace of %zu bytes required, %zu given", need,
+                    workspace ? workspace_bytes : (size_t)0);
+
+    const int nQ = Sq / BQ, nK = Sk / BK;
+    const bool bcast_b = mask_strides[0] == 0 || B == 1;
+    const bool bcast_h = mask_strides[1] == 0 || H == 1;
+    // An output dimension may be folded (stride 0) only where every plane holds the same result.
+    const int64_t ob[4] = {full_ids_strides[0], full_lens_strides[0], part_ids_strides[0], part_lens_strides[0]};
+    const int64_t oh[4] = {full_ids_strides[1], full_lens_strides[1], part_ids_strides[1], part_lens_strides[1]};
+    int zb = 0, zh = 0;
+    for (int i = 0; i < 4; i++) {
+        zb += ob[i] == 0;
+        zh += oh[i] == 0;
+    }
+    if (B > 1 && zb != 0 && (zb != 4 || !bcast_b))
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_classify: output batch stride 0 needs a batch-broadcast mask and must be 0 on all four outputs");
+    if (H > 1 && zh != 0 && (zh != 4 || !bcast_h))
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_classify: output head stride 0 needs a head-broadcast mask and must be 0 on all four outputs");
+
+    sa::ClassifyParams cp{};
+    cp.mask = mask;
+    cp.sb = mask_strides[0];
+    cp.sh = mask_strides[1];
+    cp.sq = mask_strides[2];
+    cp.sk = mask_strides[3];
+    cp.cls = static_cast<uint8_t *>(workspace);
+    cp.uB = bcast_b ? 1 : B;
+    cp.uH = bcast_h ? 1 : H;
+    cp.Sq = Sq;
+    cp.Sk = Sk;
+    cp.BQ = BQ;
+    cp.BK = BK;
+    cp.nQ = nQ;
+    cp.nK = nK;
+    cp.lbk = log2_exact(BK);
+    if (nQ > 65535 || (int64_t)cp.uB * cp.uH > 65535)
+        return fail(SA_ERR_UNSUPPORTED, "sa_mask_classify: more than 65535 Q tiles or distinct mask planes");
+
+    // Wide kernel: 16-byte loads along a contiguous, aligned key dimension; a tile spans 1..64 lanes.
+    const bool wide = cp.lbk >= 4 && BK <= 1024 && (cp.sk == 1 || Sk == 1) && aligned(mask, 16) && cp.sq % 16 == 0 &&
+                      (cp.uB == 1 || cp.sb % 16 == 0) && (cp.uH == 1 || cp.sh % 16 == 0);
+    hipError_t e = sa::launch_classify(cp, wide, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_mask_classify: classify launch failed: %s", hipGetErrorString(e));
+
+    sa::CompactParams kp{};
+    kp.cls = cp.cls;
+    kp.uH = cp.uH;
+    kp.bcast_b = bcast_b;
+    kp.bcast_h = bcast_h;
+    kp.oB = (B > 1 && zb == 4) ? 1 : B;
+    kp.oH = (H > 1 && zh == 4) ? 1 : H;
+    kp.nQ = nQ;
+    kp.nK = nK;
+    kp.full_ids = full_ids;
+    kp.full_lens = full_lens;
+    kp.part_ids = part_ids;
+    kp.part_lens = part_lens;
+    for (int i = 0; i < 4; i++) {
+        kp.fis[i] = full_ids_strides[i];
+        kp.pis[i] = part_ids_strides[i];
+    }
+    for (int i = 0; i < 3; i++) {
+        kp.fls[i] = full_lens_strides[i];
+        kp.pls[i] = part_lens_strides[i];
+    }
+    e = sa::launch_compact(kp, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_mask_classify: compaction launch failed: %s", hipGetErrorString(e));
+    return SA_OK;
+}
+
+int sa_sparse_attention_fwd(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                            const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
+                            const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
+                            const int64_t full_ids_strides[4], const int32_t *full_lens,
+                            const int64_t full_lens_strides[3], const int32_t *part_ids,
+                            const int64_t part_ids_strides[4], const int32_t *part_lens,
+                            const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int D, int BQ, int BK,
+                            int dtype, float sm_scale_log2, void *stream) {
+    g_error[0] = 0;
+    if (!q || !k || !v || !o || !mask || !q_strides || !k_strides || !v_strides || !o_strides || !mask_strides ||
+        !full_ids || !full_ids_strides || !full_lens || !full_lens_strides || !part_ids || !part_ids_strides ||
+        !part_lens || !part_lens_strides)
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd: null pointer argument");
+    if (const int rc = check_tiling(B, H, Sq, Sk, BQ, BK)) return rc;
+    if (D <= 0) return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd: D must be positive (got %d)", D);
+    if (!(sm_scale_log2 > 0.f) || !(sm_scale_log2 < 3.0e38f))
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd: sm_scale_log2 must be positive and finite");
+    if (dtype != SA_DTYPE_BF16 && dtype != SA_DTYPE_FP16)
+        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: dtype code %d (supported: 0 = bf16, 1 = fp16)", dtype);
+    if (D != 64 && D != 128) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: head dim %d (supported: 64, 128)", D);
+    if (BQ != 32 && BQ != 64 && BQ != 128)
+        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: BLOCK_Q %d (supported: 32, 64, 128)", BQ);
+    const int lbk = log2_exact(BK);
+    if (lbk < 4) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: BLOCK_K %d (supported: powers of two >= 16)", BK);
+    const int64_t *st[4] = {q_strides, k_strides, v_strides, o_strides};
+    const void *ptr[4] = {q, k, v, o};
+    const char *name[4] = {"q", "k", "v", "o"};
+    for (int t = 0; t < 4; t++) {
+        if (st[t][3] != 1 && D != 1)
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: %s must be contiguous in its last dimension (stride %lld)", name[t], (long long)st[t][3]);
+        if (!aligned(ptr[t], 16) || st[t][0] % 8 || st[t][1] % 8 || st[t][2] % 8)
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: %s needs a 16-byte aligned base and strides that are multiples of 8 elements", name[t]);
+    }
+    if (o_strides[2] == 0 || (B > 1 && o_strides[0] == 0) || (H > 1 && o_strides[1] == 0))
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd: o must not alias itself (zero stride)");
+    if ((int64_t)B * H * (Sq / BQ) > 0x7fffffffLL)
+        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: more than 2^31-1 workgroups");
+
+    sa::FwdParams fp{};
+    fp.q = static_cast<const uint16_t *>(q);
+    fp.k = static_cast<const uint16_t *>(k);
+    fp.v = static_cast<const uint16_t *>(v);
+    fp.o = static_cast<uint16_t *>(o);
+    fp.mask = mask;
+    fp.full_ids = full_ids;
+    fp.full_lens = full_lens;
+    fp.part_ids = part_ids;
+    fp.part_lens = part_lens;
+    for (int i = 0; i < 3; i++) {
+        fp.qs[i] = q_strides[i];
+        fp.ks[i] = k_strides[i];
+        fp.vs[i] = v_strides[i];
+        fp.os[i] = o_strides[i];
+        fp.fls[i] = full_lens_strides[i];
+        fp.pls[i] = part_lens_strides[i];
+    }
+    for (int i = 0; i < 4; i++) {
+        fp.ms[i] = mask_strides[i];
+        fp.fis[i] = full_ids_strides[i];
+        fp.pis[i] = part_ids_strides[i];
+    }
+    fp.B = B;
+    fp.H = H;
+    fp.Sq = Sq;
+    fp.Sk = Sk;
+    fp.nQ = Sq / BQ;
+    fp.BK = BK;
+    fp.lbk = lbk;
+    fp.mask_vec4 = (mask_strides[3] == 1 && aligned(mask, 4) && mask_strides[0] % 4 == 0 && mask_strides[1] % 4 == 0 &&
+                    mask_strides[2] % 4 == 0)
+                       ? 1
+                       : 0;
+    fp.scale = sm_scale_log2;
+    const hipError_t e = sa::launch_fwd(fp, dtype, D, BQ, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_fwd: launch failed: %s", hipGetErrorString(e));
+    return SA_OK;
+}
+
+}  // extern "C"

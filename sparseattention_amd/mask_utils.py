@@ -1,0 +1,106 @@
+"""Mask preprocessing: which (Q tile, KV tile) pairs are full, partial or empty.
+
+Mirrors the interface of the reference's ``sparseattention/mask_utils.py``:
+``MaskMetadata`` (:6-11), ``compute_mask_slow`` (:14-44), ``compute_mask_kernel`` (:85-107).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from . import _native
+
+
+@dataclass
+class MaskMetadata:
+    """Per-Q-tile index lists.  Field names and order follow mask_utils.py:6-11.
+
+    ``unmasked_kv_ids`` int32 [B,H,Sq/BQ,Sk/BK]: ascending indices of KV tiles whose mask tile is all True;
+    ``unmasked_lens``  int32 [B,H,Sq/BQ]: how many leading slots of it are valid;
+    ``masked_kv_ids`` / ``masked_lens``: the same for tiles with some but not all entries True.
+    Slots past the count hold unspecified values.
+    """
+
+    unmasked_kv_ids: torch.Tensor
+    unmasked_lens: torch.Tensor
+    masked_kv_ids: torch.Tensor
+    masked_lens: torch.Tensor
+
+
+def _check_mask(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int):
+    if mask.dim() != 4:
+        raise ValueError(f"mask must be [B,H,Sq,Sk] (got {tuple(mask.shape)}); use mask.expand(B,H,Sq,Sk)")
+    B, H, Sq, Sk = mask.shape
+    # the reference asserts these (mask_utils.py:18-20, :89-90)
+    assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
+    assert Sq % BLOCK_Q == 0, "Sq must be a multiple of BLOCK_Q"
+    assert Sk % BLOCK_K == 0, "Sk must be a multiple of BLOCK_K"
+    return B, H, Sq, Sk
+
+
+def compute_mask_slow(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int) -> MaskMetadata:
+    """Specification of the classification, in plain torch on the mask's own device.
+
+    Same results as the reference's loop (mask_utils.py:27-42) without the per-tile Python
+    iterations: a tile whose popcount equals BLOCK_Q*BLOCK_K is listed as unmasked, one with a
+    positive popcount as masked, indices ascending.  Slots past the count are filled with -1.
+    """
+    B, H, Sq, Sk = _check_mask(mask, BLOCK_Q, BLOCK_K)
+    nQ, nK = Sq // BLOCK_Q, Sk // BLOCK_K
+    # broadcast dimensions hold one distinct plane: count it once, expand the result
+    uniq = mask[:1] if mask.stride(0) == 0 else mask
+    uniq = uniq[:, :1] if mask.stride(1) == 0 else uniq
+    counts = uniq.reshape(uniq.shape[0], uniq.shape[1], nQ, BLOCK_Q, nK, BLOCK_K).sum(dim=(3, 5), dtype=torch.int64)
+    full = counts == BLOCK_Q * BLOCK_K
+    part = (counts > 0) & ~full
+
+    def compact(flags):
+        lens = flags.sum(-1).to(torch.int32)
+        order = torch.sort((~flags).to(torch.uint8), dim=-1, stable=True).indices.to(torch.int32)
+        pos = torch.arange(nK, device=mask.device, dtype=torch.int32)
+        ids = torch.where(pos < lens[..., None], order, torch.full_like(order, -1))
+        return ids.expand(B, H, nQ, nK), lens.expand(B, H, nQ)
+
+    fid, fl = compact(full)
+    pid, pl = compact(part)
+    return MaskMetadata(fid, fl, pid, pl)
+
+
+def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int) -> MaskMetadata:
+    """Classify the mask's tiles on the GPU (replaces mask_utils.py:85-107).
+
+    ``mask``: bool [B,H,Sq,Sk] on a ROCm device, any strides.  Dimensions that are broadcast in
+    ``mask`` (stride 0, e.g. from ``mask.expand(B,H,Sq,Sk)``) are classified once and the returned
+    tensors are broadcast views over them, so every ``[b,h]`` plane reads the same values the
+    reference would have written there.
+    """
+    B, H, Sq, Sk = _check_mask(mask, BLOCK_Q, BLOCK_K)
+    if not mask.is_cuda:
+        raise RuntimeError("compute_mask_kernel needs the mask on a ROCm GPU; compute_mask_slow runs anywhere")
+    lib = _native.load()
+    nQ, nK = Sq // BLOCK_Q, Sk // BLOCK_K
+    uB = 1 if (mask.stride(0) == 0 or B == 1) else B
+    uH = 1 if (mask.stride(1) == 0 or H == 1) else H
+    dev = mask.device
+    with torch.cuda.device(dev):
+        fid = torch.empty(uB, uH, nQ, nK, dtype=torch.int32, device=dev)
+        pid = torch.empty(uB, uH, nQ, nK, dtype=torch.int32, device=dev)
+        fl = torch.empty(uB, uH, nQ, dtype=torch.int32, device=dev)
+        pl = torch.empty(uB, uH, nQ, dtype=torch.int32, device=dev)
+        fid, pid = fid.expand(B, H, nQ, nK), pid.expand(B, H, nQ, nK)
+        fl, pl = fl.expand(B, H, nQ), pl.expand(B, H, nQ)
+        ms = _native.strides(mask.stride())
+        need = lib.sa_mask_classify_workspace_bytes(ms, B, H, Sq, Sk, BLOCK_Q, BLOCK_K)
+        workspace = torch.empty(max(int(need), 1), dtype=torch.uint8, device=dev)
+        rc = lib.sa_mask_classify(
+            mask.data_ptr(), ms, B, H, Sq, Sk, BLOCK_Q, BLOCK_K,
+            fid.data_ptr(), _native.strides(fid.stride()), fl.data_ptr(), _native.strides(fl.stride()),
+            pid.data_ptr(), _native.strides(pid.stride()), pl.data_ptr(), _native.strides(pl.stride()),
+            workspace.data_ptr(), workspace.numel(), torch.cuda.current_stream(dev).cuda_stream,
+        )
+        _native.check(rc)
+        # the kernels run on the current stream; the caching allocator may hand this block out again
+        # only to work queued after them on the same stream, so dropping the reference here is safe
+        del workspace
+    return MaskMetadata(fid, fl, pid, pl)

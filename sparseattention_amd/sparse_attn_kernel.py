@@ -1,0 +1,71 @@
+"""Block-sparse attention forward (replaces the reference's ``sparseattention/sparse_attn_kernel.py``)."""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _native
+from .mask_utils import MaskMetadata, compute_mask_kernel
+
+_DTYPES = {torch.bfloat16: _native.SA_DTYPE_BF16, torch.float16: _native.SA_DTYPE_FP16}
+
+
+def _kernel_ready(t: torch.Tensor) -> torch.Tensor:
+    """The kernels want a unit stride in D, 16-byte aligned rows; copy only when that does not hold."""
+    ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in t.stride()[:-1])
+    return t if ok else t.contiguous()
+
+
+def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor, BLOCK_Q, BLOCK_K,
+                     mask_metadata: MaskMetadata | None = None) -> torch.Tensor:
+    """softmax(q kᵀ / sqrt(D) + (mask ? 0 : -inf)) v, skipping KV tiles the mask empties.
+
+    Signature and meaning follow sparse_attn_kernel.py:149-185: ``q`` [B,H,Sq,D], ``k``/``v``
+    [B,H,Sk,D] (bf16 or fp16, on a ROCm GPU), ``mask`` bool broadcastable to [B,H,Sq,Sk] with
+    True = attend, tile sizes ``BLOCK_Q`` x ``BLOCK_K``, and optionally the metadata from
+    :func:`compute_mask_kernel` so that preprocessing is paid once for many calls.
+    Returns ``o`` with q's shape, dtype and strides.
+    """
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("q, k, v must be [B,H,S,D]")
+    B, H, Sq, D = q.shape
+    Sk = k.shape[-2]
+    if k.shape != (B, H, Sk, D) or v.shape != (B, H, Sk, D):
+        raise ValueError(f"k/v shapes {tuple(k.shape)}/{tuple(v.shape)} do not match q {tuple(q.shape)}")
+    if not q.is_cuda:
+        raise RuntimeError("sparse_attention needs q, k, v on a ROCm GPU; there is no CPU path")
+    if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise TypeError(f"q, k, v must share dtype bfloat16 or float16 (got {q.dtype}, {k.dtype}, {v.dtype})")
+    sm_scale = D ** (-0.5) * 1 / math.log(2)  # exp2 replaces exp (sparse_attn_kernel.py:152)
+
+    mask = mask.expand(B, H, Sq, Sk)
+
+    if mask_metadata is None:
+        mask_metadata = compute_mask_kernel(mask, BLOCK_Q, BLOCK_K)
+    fid, fl = mask_metadata.unmasked_kv_ids, mask_metadata.unmasked_lens
+    pid, pl = mask_metadata.masked_kv_ids, mask_metadata.masked_lens
+    nQ, nK = Sq // BLOCK_Q, Sk // BLOCK_K
+    for name, t, shape in (("unmasked_kv_ids", fid, (B, H, nQ, nK)), ("masked_kv_ids", pid, (B, H, nQ, nK)),
+                           ("unmasked_lens", fl, (B, H, nQ)), ("masked_lens", pl, (B, H, nQ))):
+        if tuple(t.shape) != shape or t.dtype != torch.int32 or t.device != q.device:
+            raise ValueError(f"mask_metadata.{name}: expected int32 {shape} on {q.device}, got {t.dtype} {tuple(t.shape)} on {t.device}")
+    assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
+    if mask.device != q.device:
+        raise ValueError("mask must be on the same device as q")
+
+    qc, kc, vc = _kernel_ready(q), _kernel_ready(k), _kernel_ready(v)
+    o = torch.empty_like(qc)
+    lib = _native.load()
+    S = _native.strides
+    with torch.cuda.device(q.device):
+        rc = lib.sa_sparse_attention_fwd(
+            qc.data_ptr(), S(qc.stride()), kc.data_ptr(), S(kc.stride()), vc.data_ptr(), S(vc.stride()),
+            o.data_ptr(), S(o.stride()), mask.data_ptr(), S(mask.stride()),
+            fid.data_ptr(), S(fid.stride()), fl.data_ptr(), S(fl.stride()),
+            pid.data_ptr(), S(pid.stride()), pl.data_ptr(), S(pl.stride()),
+            B, H, Sq, Sk, D, int(BLOCK_Q), int(BLOCK_K), _DTYPES[q.dtype], sm_scale,
+            torch.cuda.current_stream(q.device).cuda_stream,
+        )
+    _native.check(rc)
+    return o
