@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Benchmark of the block-sparse attention forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-sweep] [--no-cpu]
+
+A step is one forward pass (sa_sparse_attention_fwd) over the headline workload: causal bool mask
+passed as a tensor, B=8 H=32 S=4096 D=128 bf16, tiles 128x32, inputs and the precomputed tile lists
+resident in HBM (the reference also excludes preprocessing from the forward time and reports it
+separately, test_attn.py:38,65,68).  Prints ONE JSON line.
+
+  value      effective TFLOP/s by the reference's convention: 4*B*H*Sq*Sk*D * mean(mask) / time
+             (test_attn.py:84, :108-111)
+  roofline   the forward kernel against the dense bf16 MFMA peak, counting executed tiles only:
+             (full + partial tiles) * 4*BQ*BK*D flop per launch / mean launch duration (HIP events)
+  mask_classify   the preprocessing kernels on a 1 GiB mask against the HBM peak
+  across_p   the same forward on random block masks of sparsity p, a dense mask and the causal one
+  cpu_baseline / cpu_sdpa_baseline   the CPU oracle and torch's masked SDPA on a bounded sample
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak, TFLOP/s
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E peak, GB/s
+
+B, H, S, D = 8, 32, 4096, 128
+BQ, BK = 128, 32
+FLOP_PER_TILE = 4 * BQ * BK * D
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-sweep", action="store_true", help="skip the across-p table")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--no-classify", action="store_true", help="skip the mask-classification timing")
+    return ap.parse_args()
+
+
+def time_launches(fn, steps, warmup):
+    """Wall time per step (host clock, synchronised on both sides) and mean per-launch duration from HIP
+    events recorded on the stream the kernel is launched on (torch's current stream)."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        fn()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev_ms = sum(s.elapsed_time(e) for s, e in zip(starts, ends)) / steps
+    return wall_ms, ev_ms
+
+
+def forward_case(name, mask2d, q, k, v, steps, warmup):
+    import torch
+    from sparseattention_amd import compute_mask_kernel, sparse_attention
+
+    me = mask2d[None, None].expand(B, H, S, S)
+    md = compute_mask_kernel(me, BQ, BK)
+    tiles_plane = int(md.unmasked_lens[0, 0].sum()) + int(md.masked_lens[0, 0].sum())
+    partial_plane = int(md.masked_lens[0, 0].sum())
+    frac = float(mask2d.float().mean())
+    wall_ms, ev_ms = time_launches(lambda: sparse_attention(q, k, v, me, BQ, BK, mask_metadata=md), steps, warmup)
+    executed = tiles_plane * B * H * FLOP_PER_TILE
+    useful = 4 * B * H * S * S * D * frac
+    return {
+        "mask": name,
+        "fraction_unmasked": round(frac, 5),
+        "executed_tile_fraction": round(tiles_plane / ((S // BQ) * (S // BK)), 5),
+        "partial_tiles_per_plane": partial_plane,
+        "ms": round(wall_ms, 4),
+        "kernel_ms": round(ev_ms, 4),
+        "effective_tflops": round(useful / (wall_ms * 1e-3) / 1e12, 2),
+        "executed_tflops": round(executed / (ev_ms * 1e-3) / 1e12, 2),
+        "_executed_flop": executed,
+        "_useful_flop": useful,
+    }
+
+
+def classify_case(steps, warmup):
+    """Preprocessing on the largest single-plane mask of the configurations (S=32768, 1 GiB)."""
+    import torch
+    from sparseattention_amd import _native, workloads as W
+
+    lib = _native.load()
+    Sbig = 32768
+    mask = W.composed_mask(Sbig, device="cuda")[None, None]
+    nQ, nK = Sbig // BQ, Sbig // BK
+    fid = torch.empty(1, 1, nQ, nK, dtype=torch.int32, device="cuda")
+    pid = torch.empty_like(fid)
+    fl = torch.empty(1, 1, nQ, dtype=torch.int32, device="cuda")
+    pl = torch.empty_like(fl)
+    ms = _native.strides(mask.stride())
+    need = lib.sa_mask_classify_workspace_bytes(ms, 1, 1, Sbig, Sbig, BQ, BK)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    st = _native.strides
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def run():
+        rc = lib.sa_mask_classify(mask.data_ptr(), ms, 1, 1, Sbig, Sbig, BQ, BK, fid.data_ptr(), st(fid.stride()),
+                                  fl.data_ptr(), st(fl.stride()), pid.data_ptr(), st(pid.stride()), pl.data_ptr(),
+                                  st(pl.stride()), ws.data_ptr(), need, stream)
+        _native.check(rc)
+
+    wall_ms, ev_ms = time_launches(run, steps, warmup)
+    nbytes = Sbig * Sbig + nQ * (2 * nK + 2) * 4  # mask read once + lists and counts written
+    return {
+        "workload": "sa_mask_classify on the composed mask, bool [32768,32768] = 1 GiB, tiles 128x32",
+        "ms": round(ev_ms, 4),
+        "roofline": {"bound": "hbm", "achieved": round(nbytes / (ev_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(nbytes / (ev_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None},
+    }
+
+
+def classify_small_case(steps, warmup):
+    """Preprocessing of the headline mask itself ([4096,4096] = 16 MiB): launch-latency bound."""
+    import torch
+    from sparseattention_amd import compute_mask_kernel, workloads as W
+
+    me = W.causal_mask(S, "cuda")[None, None].expand(B, H, S, S)
+    wall_ms, ev_ms = time_launches(lambda: compute_mask_kernel(me, BQ, BK), steps, warmup)
+    return {"workload": "compute_mask_kernel on the causal mask [4096,4096] = 16 MiB (latency bound)", "ms": round(ev_ms, 4)}
+
+
+def cpu_baselines():
+    """Bounded CPU legs on the host cores: (a) the C oracle (a port of the reference algorithm),
+    (b) torch's masked SDPA on CPU tensors, the reference's own check path (test_attn.py:40)."""
+    import torch
+    import torch.nn.functional as F
+
+    import oracle
+    from sparseattention_amd import workloads as W
+
+    mask = W.causal_mask(S)
+    frac = float(mask.float().mean())
+    out = {}
+    # (a) oracle: one (b,h) plane of the workload
+    hp = 2
+    q, k, v = W.qkv(1, hp, S, D, torch.bfloat16, seed=0)
+    qf, kf, vf = (t.float().numpy() for t in (q, k, v))
+    m4 = mask.numpy()[None, None]
+    meta = oracle.classify(m4.repeat(hp, 1), BQ, BK)
+    t0 = time.perf_counter()
+    oracle.forward(qf, kf, vf, m4, BQ, BK, meta=meta, p_round=1)
+    dt = time.perf_counter() - t0
+    useful = 4 * 1 * hp * S * S * D * frac
+    out["cpu_baseline"] = {
+        "value": round(useful / dt / 1e12, 5), "unit": "TFLOP/s", "cores": oracle.max_threads(), "kind": "port",
+        "sample": f"C oracle two-pass forward (oracle/sparse_oracle.c, OpenMP) on B=1 H={hp} of the workload "
+                  f"(causal S={S} D={D}, bf16 inputs widened to fp32, tiles {BQ}x{BK}): {dt:.2f} s, effective TFLOP/s",
+        "ms_full_workload_extrapolated": round(dt * 1e3 * B * H / hp, 1),
+    }
+    # (b) torch SDPA with the tensor mask on CPU
+    hs = 8
+    q, k, v = W.qkv(1, hs, S, D, torch.bfloat16, seed=0)
+    F.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        F.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+        ts.append(time.perf_counter() - t0)
+    dt = sorted(ts)[1]
+    useful = 4 * 1 * hs * S * S * D * frac
+    out["cpu_sdpa_baseline"] = {
+        "value": round(useful / dt / 1e12, 5), "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "library",
+        "sample": f"torch {torch.__version__} F.scaled_dot_product_attention(q,k,v,attn_mask=mask) on CPU bf16 tensors, "
+                  f"B=1 H={hs} of the workload, median of 3: {dt:.3f} s, effective TFLOP/s",
+        "ms_full_workload_extrapolated": round(dt * 1e3 * B * H / hs, 1),
+        "host_cpu_count": os.cpu_count(),
+    }
+    return out
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); the path has no multi-GPU leg.",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no ROCm GPU visible; the forward path has no CPU fallback.", file=sys.stderr)
+        sys.exit(2)
+    from sparseattention_amd import _native, workloads as W
+
+    _native.load()
+    torch.cuda.set_device(0)
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=0, device="cuda")
+
+    head = forward_case("causal", W.causal_mask(S, "cuda"), q, k, v, args.steps, args.warmup)
+    achieved = head["_executed_flop"] / (head["kernel_ms"] * 1e-3) / 1e12
+    result = {
+        "metric": "effective TFLOP/s of the block-sparse forward (4*B*H*S*S*D*mean(mask)/time), B8 H32 S4096 D128 bf16",
+        "value": head["effective_tflops"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: causal bool mask [4096,4096] passed as a tensor, B=8 H=32 S=4096 D=128 bf16, "
+                               "q/k/v ~ N(0,1), tiles BLOCK_Q=128 BLOCK_K=32, tile lists precomputed",
+                   "executed_tiles_per_plane": int(head["_executed_flop"] // (B * H * FLOP_PER_TILE)),
+                   "partial_tiles_per_plane": head["partial_tiles_per_plane"]},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "kernel": "sparse_fwd_kernel", "kernel_ms": head["kernel_ms"],
+                     "flop_per_launch": head["_executed_flop"]},
+    }
+    if not args.no_sweep:
+        rows = [head]
+        sweep_steps, sweep_warm = max(5, args.steps // 5), max(2, args.warmup // 3)
+        rows.append(forward_case("dense (all True)", torch.ones(S, S, dtype=torch.bool, device="cuda"), q, k, v,
+                                 sweep_steps, sweep_warm))
+        for p in (0.25, 0.5, 0.75, 0.9):
+            m = W.random_block_mask(S, 128, p, seed=int(p * 100), device="cuda")
+            rows.append(forward_case(f"random blocks p={p}", m, q, k, v, sweep_steps, sweep_warm))
+        result["across_p"] = [{kk: vv for kk, vv in r.items() if not kk.startswith("_")} for r in rows]
+    if not args.no_classify:
+        result["mask_classify"] = classify_case(max(10, args.steps // 2), max(3, args.warmup // 2))
+        result["mask_classify_headline"] = classify_small_case(max(10, args.steps // 2), max(3, args.warmup // 2))
+    del q, k, v
+    if not args.no_cpu:
+        result.update(cpu_baselines())
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

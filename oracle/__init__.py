@@ -56,8 +56,21 @@ def _load():
         [f32p, f32p, f32p, f32p, u8p, i64p, i32p, i32p, i32p, i32p] + [ctypes.c_int] * 7 + [ctypes.c_float, ctypes.c_int]
     )
     lib.oracle_max_threads.restype = ctypes.c_int
+    for fn in (lib.oracle_round_bf16, lib.oracle_round_fp16):
+        fn.restype = ctypes.c_float
+        fn.argtypes = [ctypes.c_float]
     _lib = lib
     return lib
+
+
+def round_bf16(x: float) -> float:
+    """fp32 -> nearest bf16 -> fp32, as the C oracle rounds P."""
+    return float(_load().oracle_round_bf16(x))
+
+
+def round_fp16(x: float) -> float:
+    """fp32 -> nearest fp16 -> fp32, as the C oracle rounds P."""
+    return float(_load().oracle_round_fp16(x))
 
 
 def max_threads() -> int:

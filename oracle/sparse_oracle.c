@@ -73,6 +73,10 @@ static inline float round_to_fp16(float x) {
     return x < 0 ? -r : r;
 }
 
+/* Exported so that tests can compare the two rounding helpers with torch's casts directly. */
+float oracle_round_bf16(float x) { return round_to_bf16(x); }
+float oracle_round_fp16(float x) { return round_to_fp16(x); }
+
 /*
  * Tile classification.  mask is addressed as mask[b*ms[0] + h*ms[1] + q*ms[2] + k*ms[3]]
  * (strides in bytes == elements, any value including 0); a byte != 0 means "attend".

@@ -1,0 +1,131 @@
+"""The C-ABI library: it loads, exports every symbol the header declares, and rejects bad
+arguments on the host before any kernel is launched (so these run without a GPU)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from sparseattention_amd import _native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "sparseattn.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_library_agree():
+    names = declared_functions()
+    assert names, "no functions found in the header"
+    lib = _native.load()
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in sparseattn.h but not exported"
+    assert sorted(_native.EXPORTS) == names
+    assert lib.sa_abi_version() == _native.SA_ABI_VERSION
+    header = open(HEADER).read()
+    assert f"#define SA_ABI_VERSION {_native.SA_ABI_VERSION}" in header
+    for name in ("SA_ERR_INVALID_ARGUMENT", "SA_ERR_UNSUPPORTED", "SA_ERR_WORKSPACE", "SA_ERR_HIP"):
+        assert re.search(rf"{name}\s*=\s*{getattr(_native, name)}\b", header)
+
+
+def test_every_entry_point_cites_the_reference_interface_it_replaces():
+    text = open(HEADER).read()
+    assert "mask_utils.py:85-107" in text and "sparse_attn_kernel.py:149-185" in text
+
+
+FAKE = 0x1000  # never dereferenced: every call below must fail validation first
+S4 = _native.strides((0, 0, 64, 1))
+S3 = _native.strides((0, 0, 1))
+I4 = _native.strides((0, 0, 2, 1))
+
+
+def classify(mask=FAKE, ms=S4, B=1, H=1, Sq=64, Sk=64, BQ=32, BK=32, ws=FAKE, ws_bytes=1 << 20, out=FAKE, ids_strides=I4):
+    lib = _native.load()
+    return lib.sa_mask_classify(mask, ms, B, H, Sq, Sk, BQ, BK, out, ids_strides, out, S3, out, ids_strides, out, S3, ws,
+                                ws_bytes, None)
+
+
+def fwd(q=FAKE, D=128, BQ=128, BK=32, dtype=0, Sq=256, Sk=256, scale=0.1, qs=None, B=1, H=1):
+    lib = _native.load()
+    qs = qs or _native.strides((Sq * D, Sq * D, D, 1))
+    return lib.sa_sparse_attention_fwd(q, qs, FAKE, qs, FAKE, qs, FAKE, qs, FAKE, _native.strides((0, 0, Sk, 1)),
+                                       FAKE, I4, FAKE, S3, FAKE, I4, FAKE, S3, B, H, Sq, Sk, D, BQ, BK, dtype, scale, None)
+
+
+def last_error():
+    return _native.load().sa_last_error().decode()
+
+
+def test_classify_rejects_bad_arguments():
+    assert classify(mask=None) == _native.SA_ERR_INVALID_ARGUMENT and "null" in last_error()
+    assert classify(out=None) == _native.SA_ERR_INVALID_ARGUMENT
+    assert classify(Sq=65) == _native.SA_ERR_INVALID_ARGUMENT and "BLOCK_Q" in last_error()
+    assert classify(Sk=100) == _native.SA_ERR_INVALID_ARGUMENT and "BLOCK_K" in last_error()
+    assert classify(BQ=0) == _native.SA_ERR_INVALID_ARGUMENT
+    assert classify(B=0) == _native.SA_ERR_INVALID_ARGUMENT
+    assert classify(ws=None) == _native.SA_ERR_WORKSPACE
+    assert classify(ws_bytes=3) == _native.SA_ERR_WORKSPACE and "4 bytes required" in last_error()
+    # folded output planes need a broadcast mask
+    assert classify(B=2, ms=_native.strides((4096, 0, 64, 1))) == _native.SA_ERR_INVALID_ARGUMENT
+
+
+def test_workspace_size_counts_distinct_planes_only():
+    lib = _native.load()
+    f = lib.sa_mask_classify_workspace_bytes
+    assert f(_native.strides((0, 0, 4096, 1)), 8, 32, 4096, 4096, 128, 32) == 32 * 128
+    assert f(_native.strides((1 << 24, 0, 4096, 1)), 8, 32, 4096, 4096, 128, 32) == 8 * 32 * 128
+    assert f(_native.strides((1 << 29, 1 << 24, 4096, 1)), 8, 32, 4096, 4096, 128, 32) == 8 * 32 * 32 * 128
+    assert f(_native.strides((0, 0, 4096, 1)), 8, 32, 4096, 4096, 100, 32) == 0
+
+
+def test_forward_rejects_bad_arguments():
+    assert fwd(q=None) == _native.SA_ERR_INVALID_ARGUMENT
+    assert fwd(Sq=200) == _native.SA_ERR_INVALID_ARGUMENT
+    assert fwd(scale=0.0) == _native.SA_ERR_INVALID_ARGUMENT
+    assert fwd(scale=float("nan")) == _native.SA_ERR_INVALID_ARGUMENT
+    assert fwd(D=96) == _native.SA_ERR_UNSUPPORTED and "head dim" in last_error()
+    assert fwd(BQ=16, Sq=256) == _native.SA_ERR_UNSUPPORTED and "BLOCK_Q" in last_error()
+    assert fwd(BK=8) == _native.SA_ERR_UNSUPPORTED and "BLOCK_K" in last_error()
+    assert fwd(BK=4, Sk=252, Sq=256) == _native.SA_ERR_UNSUPPORTED
+    assert fwd(dtype=7) == _native.SA_ERR_UNSUPPORTED and "dtype" in last_error()
+    assert fwd(q=FAKE + 2) == _native.SA_ERR_UNSUPPORTED and "aligned" in last_error()
+    assert fwd(qs=_native.strides((256 * 128, 256 * 128, 128, 2))) == _native.SA_ERR_UNSUPPORTED
+    assert fwd(qs=_native.strides((256 * 128, 256 * 128, 132, 1))) == _native.SA_ERR_UNSUPPORTED
+
+
+def test_python_wrappers_refuse_to_run_without_a_gpu_tensor():
+    from sparseattention_amd import compute_mask_kernel, sparse_attention
+
+    m = torch.ones(1, 1, 64, 64, dtype=torch.bool)
+    with pytest.raises(RuntimeError, match="GPU"):
+        compute_mask_kernel(m, 32, 32)
+    q = torch.zeros(1, 1, 64, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        sparse_attention(q, q, q, m, 32, 32)
+    with pytest.raises(AssertionError):
+        compute_mask_kernel(m, 48, 32)  # same assertion as mask_utils.py:89
+
+
+def test_check_maps_codes_to_exceptions():
+    assert classify(Sq=65) == _native.SA_ERR_INVALID_ARGUMENT
+    with pytest.raises(ValueError, match="BLOCK_Q"):
+        _native.check(_native.SA_ERR_INVALID_ARGUMENT)
+    assert fwd(D=96) == _native.SA_ERR_UNSUPPORTED
+    with pytest.raises(_native.SparseAttnError) as ei:
+        _native.check(_native.SA_ERR_UNSUPPORTED)
+    assert ei.value.code == _native.SA_ERR_UNSUPPORTED
+
+
+def test_product_code_never_touches_the_oracle():
+    pkg = os.path.join(ROOT, "sparseattention_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"^\s*(import|from)\s+oracle\b", text, flags=re.M), f
+                assert "liboracle" not in text, f
