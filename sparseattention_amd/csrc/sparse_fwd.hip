@@ -20,11 +20,14 @@
 //                   16-key MFMA step, so P never leaves registers; the matching A operand is read
 //                   from row-major V in LDS with the transposing ds_read_b64_tr_b16.
 //
-// LDS: two buffers each for K and V (64 rows per buffer); row pitch D*2+16 bytes for K (conflict-free
-// 16-byte reads down a column of rows) and D*2+64 for V (the four rows of a transposing read fall in
-// different bank quarters).
+// LDS: two buffers each for K and V (64 rows per buffer), filled straight from global memory
+// (global_load_lds_dwordx4, 1 KiB per wave instruction) one chunk ahead of the MFMAs.  Rows are
+// unpadded; bank conflicts are avoided by XOR-swizzling the 16-byte pieces of a row (k_swizzle,
+// v_swizzle).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 #include "kernels.h"
 
@@ -92,24 +95,44 @@ __device__ __forceinline__ float half_swap_sum(float x) {
 
 constexpr float kNegInf = -__builtin_inff();
 
+// Swizzles of the 16-byte pieces inside an LDS row.  Rows are stored unpadded (D*2 bytes) because a
+// direct global->LDS load writes 64 lanes x 16 bytes contiguously; instead the piece index is XORed
+// with a function of the row so that
+//   K: the 16 rows read together by one quarter-wave ds_read_b128 fall into 16 different bank groups,
+//   V: the 4 rows touched by one half-wave transposing read fall into 4 different 64-byte bank groups.
+template <int D>
+__device__ __forceinline__ int k_swizzle(int row) {
+    return D == 128 ? (row & 15) : ((row >> 1) & 7);
+}
+template <int D>
+__device__ __forceinline__ int v_swizzle(int row) {
+    return D == 128 ? 4 * (row & 3) : 4 * ((row >> 1) & 1);
+}
+
+// log2-domain slack before the running maximum is raised (and the accumulator rescaled).  Scores are
+// exponentiated against a reference value that may lag the true row maximum by up to this much, so
+// P stays <= 2^kMaxSlack; the final division by the row sum cancels the reference exactly.
+constexpr float kMaxSlack = 8.0f;
+
+// List entries kept in LDS per Q tile (8 KiB); longer lists are read from global memory per chunk.
+constexpr int kListCap = 2048;
+
 // MODE 0: BK = 16, MODE 1: BK = 32, MODE 2: BK >= 64 (runtime log2 in p.lbk).
 template <int DT, int D, int NW, int MODE>
 __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(const FwdParams p) {
     using E = Elem<DT>;
-    constexpr int NT = NW * 64;          // threads
-    constexpr int DV = D / 8;            // 16-byte pieces per K/V row
-    constexpr int RPP = NT / DV;         // rows staged per pass of the whole workgroup
-    constexpr int NL = 64 / RPP;         // passes per 64-row chunk
-    constexpr int KSTR = D * 2 + 16;     // LDS row pitch of K, bytes
-    constexpr int VSTR = D * 2 + 64;     // LDS row pitch of V, bytes
-    constexpr int KBUF = 64 * KSTR, VBUF = 64 * VSTR;
+    constexpr int ROWB = D * 2;                   // bytes per K/V row in LDS
+    constexpr int KBUF = 64 * ROWB, VBUF = 64 * ROWB;
+    constexpr int RPI = 1024 / ROWB;              // rows written by one wave-wide direct load (1 KiB)
+    constexpr int NLD = 64 / (RPI * NW);          // direct loads per wave per chunk, each for K and for V
+    constexpr int PPR = ROWB / 16;                // 16-byte pieces per row
     constexpr int EPC = MODE == 0 ? 4 : (MODE == 1 ? 2 : 1);  // list entries per chunk
     constexpr int LBKC = MODE == 0 ? 4 : 5;                   // log2(BK) when MODE < 2
-    static_assert(RPP >= 1 && 64 % RPP == 0, "staging layout");
+    static_assert(64 % (RPI * NW) == 0, "staging layout");
 
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    uint8_t *const ksm = smem;
-    uint8_t *const vsm = smem + 2 * KBUF;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    // [K buf 0][K buf 1][V buf 0][V buf 1][first key column of every list entry, kListCap ints]
+    int *const ent = reinterpret_cast<int *>(smem + 2 * KBUF + 2 * VBUF);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, hh = lane >> 5;
@@ -145,7 +168,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         for (int c = 0; c < D / 16; c++) qf[c] = *(const u32x4 *)(qp + 16 * c);
     }
 
-    float m_run = kNegInf;  // running row maximum, in exp2 units (score * scale)
+    float m_run = kNegInf;  // reference value of the row's exponentials, in exp2 units (score * scale)
     float l_run = 0.f;      // running row sum over this lane's half of the keys
     f32x16 acc[D / 32];
 #pragma unroll
@@ -153,25 +176,61 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
 #pragma unroll
         for (int i = 0; i < 16; i++) acc[db][i] = 0.f;
 
-    // First key column of every list entry in chunk t, plus which entries exist / are partial.
+    // ---- per-lane LDS offsets (bytes, relative to the start of a K or V buffer) -------------------
+    // K operand of step c: row 32kb + l32, piece 2c + hh, swizzled.  (2c + hh) ^ s == (2c) ^ (hh ^ s).
+    int koff[D / 16];
+    {
+        const int t = hh ^ k_swizzle<D>(l32);
+#pragma unroll
+        for (int c = 0; c < D / 16; c++) koff[c] = l32 * ROWB + 16 * ((2 * c) ^ t);
+    }
+    // V^T operand (transposing read): within each 16-lane group, lane t supplies the address of 4
+    // consecutive d of key row (t >> 2) and receives the 4 key rows of d column t.
+    int voff[D / 32];
+    {
+        const int tr_row = 4 * hh + ((lane & 15) >> 2);        // + 16kc (+8 for the second read)
+        const int x = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);  // piece within the 32-wide d block
+        const int sw = v_swizzle<D>(tr_row) >> 2;               // 16kc and 8 leave the swizzle bits alone
+#pragma unroll
+        for (int db = 0; db < D / 32; db++) voff[db] = tr_row * ROWB + 64 * (db ^ sw) + 16 * x + 8 * (lane & 1);
+    }
+    // Direct-load staging: load i of this wave fills rows [RPI*(NW*i + wave), +RPI) of the chunk; lane
+    // writes row ld_row(i), LDS piece lane % PPR, and therefore fetches the swizzled source piece.
+    const int ld_r0 = lane / PPR, ld_slot = lane % PPR;
+
+    // The Q tile's list (FULL entries, then PARTIAL entries) as first key columns, copied to LDS once:
+    // loads issued after the first barrier cannot use the scalar cache, and a vector load of an index in
+    // front of every chunk would put a full memory round trip on the critical path.
+    const bool list_in_lds = NE <= kListCap;
+    if (list_in_lds) {
+        for (int e = tid; e < NE; e += NW * 64) {
+            const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
+            ent[e] = MODE == 2 ? (idx << p.lbk) : (idx << LBKC);
+        }
+    }
+    auto entry_col = [&](int e) -> int {
+        if (list_in_lds) return ent[e];
+        const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
+        return MODE == 2 ? (idx << p.lbk) : (idx << LBKC);
+    };
+
+    // First key column of every list entry in chunk t (t < T), plus which entries exist / are partial.
     auto chunk_entries = [&](int t, int(&col)[EPC], unsigned &valid, unsigned &part) {
         valid = 0u;
         part = 0u;
         if constexpr (MODE == 2) {
             const int sh = p.lbk - 6;
             const int e = t >> sh, sub = t & ((1 << sh) - 1);
-            const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
-            col[0] = (idx << p.lbk) + (sub << 6);
+            col[0] = entry_col(e) + (sub << 6);
             valid = 1u;
             part = e >= F ? 1u : 0u;
         } else {
 #pragma unroll
             for (int j = 0; j < EPC; j++) {
                 const int e = t * EPC + j;
-                col[j] = 0;
+                // absent entries re-read the chunk's first one; their scores are discarded
+                col[j] = entry_col(e < NE ? e : t * EPC);
                 if (e < NE) {
-                    const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
-                    col[j] = idx << LBKC;
                     valid |= 1u << j;
                     if (e >= F) part |= 1u << j;
                 }
@@ -179,84 +238,76 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         }
     };
 
-    // Global -> registers for one chunk: thread covers row i*RPP + tid/DV, 16-byte piece tid%DV.
-    auto load_chunk = [&](const int(&col)[EPC], unsigned valid, u32x4(&gk)[NL], u32x4(&gv)[NL]) {
-        const int r0 = tid / DV, dv = tid % DV;
+    // Global -> LDS for one chunk, without passing through registers.
+    auto stage_chunk = [&](int buf, const int(&col)[EPC]) {
 #pragma unroll
-        for (int i = 0; i < NL; i++) {
-            const int r = i * RPP + r0;
+        for (int i = 0; i < NLD; i++) {
+            const int rbase = RPI * (NW * i + wave);  // wave-uniform
+            const int r = rbase + ld_r0;
             int j = 0, within = r;
             if constexpr (MODE != 2) {
                 j = r >> LBKC;
                 within = r & ((1 << LBKC) - 1);
             }
             int c0 = col[0];
-            bool ok = valid & 1u;
 #pragma unroll
             for (int jj = 1; jj < EPC; jj++)
-                if (j == jj) {
-                    c0 = col[jj];
-                    ok = (valid >> jj) & 1u;
-                }
+                if (j == jj) c0 = col[jj];
             const int64_t srow = c0 + within;
-            if (ok) {
-                gk[i] = *(const u32x4 *)(kbase + srow * p.ks[2] + dv * 8);
-                gv[i] = *(const u32x4 *)(vbase + srow * p.vs[2] + dv * 8);
-            } else {
-                gk[i] = u32x4{0u, 0u, 0u, 0u};
-                gv[i] = u32x4{0u, 0u, 0u, 0u};
-            }
+            const uint16_t *gk = kbase + srow * p.ks[2] + 8 * (ld_slot ^ k_swizzle<D>(r));
+            const uint16_t *gv = vbase + srow * p.vs[2] + 8 * (ld_slot ^ v_swizzle<D>(r));
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gk,
+                                             (SA_LDS void *)(smem + buf * KBUF + rbase * ROWB), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gv,
+                                             (SA_LDS void *)(smem + 2 * KBUF + buf * VBUF + rbase * ROWB), 16, 0, 0);
         }
     };
-    auto store_chunk = [&](int buf, const u32x4(&gk)[NL], const u32x4(&gv)[NL]) {
-        const int r0 = tid / DV, dv = tid % DV;
+
+    // Mask bytes of this lane's eight 4-key groups in a chunk (non-zero byte = attended key).  Called for
+    // chunks with a PARTIAL or absent entry only.  FULL entries are read too (their bytes are all set),
+    // absent entries are forced to zero: no branches, eight independent loads.
+    auto load_mask = [&](const int(&col)[EPC], unsigned valid, uint32_t(&mk)[2][4]) {
+        int64_t c[2][4];
+        uint32_t keep[2][4];
 #pragma unroll
-        for (int i = 0; i < NL; i++) {
-            const int r = i * RPP + r0;
-            *(u32x4 *)(ksm + buf * KBUF + r * KSTR + dv * 16) = gk[i];
-            *(u32x4 *)(vsm + buf * VBUF + r * VSTR + dv * 16) = gv[i];
-        }
-    };
-
-    auto compute = [&](int buf, const int(&col)[EPC], unsigned valid, unsigned part) {
-        const uint8_t *kb_ = ksm + buf * KBUF;
-        const uint8_t *vb_ = vsm + buf * VBUF;
-        const bool special = part != 0u || valid != ((1u << EPC) - 1u);  // wave-uniform
-
-        // Mask bytes for this lane's 4-key groups, fetched before the MFMAs so the latency overlaps.
-        uint32_t mk[2][4];
-        if (special) {
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                int j, within;
+                if constexpr (MODE == 0) {
+                    j = 2 * kb + (g >> 1);
+                    within = 8 * (g & 1) + 4 * hh;
+                } else if constexpr (MODE == 1) {
+                    j = kb;
+                    within = 8 * g + 4 * hh;
+                } else {
+                    j = 0;
+                    within = 32 * kb + 8 * g + 4 * hh;
+                }
+                c[kb][g] = col[j] + within;
+                keep[kb][g] = ((valid >> j) & 1u) ? 0xffffffffu : 0u;
+            }
+        if (p.mask_vec4) {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) mk[kb][g] = *(const uint32_t *)(mrow + c[kb][g]) & keep[kb][g];
+        } else {
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
-                    int j, within;
-                    if constexpr (MODE == 0) {
-                        j = 2 * kb + (g >> 1);
-                        within = 8 * (g & 1) + 4 * hh;
-                    } else if constexpr (MODE == 1) {
-                        j = kb;
-                        within = 8 * g + 4 * hh;
-                    } else {
-                        j = 0;
-                        within = 32 * kb + 8 * g + 4 * hh;
-                    }
-                    uint32_t w = 0u;  // entry absent: all four keys masked out
-                    if ((valid >> j) & 1u) {
-                        w = 0x01010101u;  // FULL entry: all four keys attended
-                        if ((part >> j) & 1u) {
-                            const int64_t c = col[j] + within;
-                            if (p.mask_vec4) {
-                                w = *(const uint32_t *)(mrow + c);
-                            } else {
-                                w = (uint32_t)mrow[c * p.ms[3]] | ((uint32_t)mrow[(c + 1) * p.ms[3]] << 8) |
-                                    ((uint32_t)mrow[(c + 2) * p.ms[3]] << 16) | ((uint32_t)mrow[(c + 3) * p.ms[3]] << 24);
-                            }
-                        }
-                    }
-                    mk[kb][g] = w;
+                    const uint8_t *m0 = mrow + c[kb][g] * p.ms[3];
+                    mk[kb][g] = ((uint32_t)m0[0] | ((uint32_t)m0[p.ms[3]] << 8) | ((uint32_t)m0[2 * p.ms[3]] << 16) |
+                                 ((uint32_t)m0[3 * p.ms[3]] << 24)) & keep[kb][g];
                 }
         }
+    };
+
+    auto compute = [&](auto buf_c, bool special, const uint32_t(&mk)[2][4]) {
+        constexpr int BUF = decltype(buf_c)::value;
+        const uint8_t *kb_ = smem + BUF * KBUF;
+        const uint8_t *vb_ = smem + 2 * KBUF + BUF * VBUF;
 
         // S^T = K . Q^T
         f32x16 s[2];
@@ -266,7 +317,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
             for (int i = 0; i < 16; i++) s[kb][i] = 0.f;
 #pragma unroll
             for (int c = 0; c < D / 16; c++) {
-                const u32x4 a = *(const u32x4 *)(kb_ + (32 * kb + l32) * KSTR + (16 * c + 8 * hh) * 2);
+                const u32x4 a = *(const u32x4 *)(kb_ + 32 * kb * ROWB + koff[c]);
                 s[kb] = E::mfma(a, qf[c], s[kb]);
             }
         }
@@ -281,17 +332,26 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
                         if (((mk[kb][g] >> (8 * j)) & 0xffu) == 0u) s[kb][4 * g + j] = kNegInf;
         }
 
-        // Online softmax in exp2 units (sparse_attn_kernel.py:47-58).
+        // Online softmax in exp2 units (sparse_attn_kernel.py:47-58), with a lagging reference value.
         float mx = kNegInf;
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
             for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[kb][i]);
-        mx = half_swap_max(mx);
-        const float m_new = fmaxf(m_run, mx * p.scale);
-        const float m_ref = m_new == kNegInf ? 0.f : m_new;  // keeps exp2(-inf - -inf) out of the picture
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
-        m_run = m_new;
+        mx = half_swap_max(mx) * p.scale;
+        const bool raise = mx > m_run + kMaxSlack;  // also true for the first finite maximum (m_run = -inf)
+        if (__builtin_amdgcn_ballot_w64(raise) != 0ull) {
+            const float m_new = raise ? mx : m_run;
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // m_new is finite wherever raise holds
+            const float a = raise ? alpha : 1.f;
+            m_run = m_new;
+            l_run *= a;
+#pragma unroll
+            for (int db = 0; db < D / 32; db++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc[db][i] *= a;
+        }
+        const float m_ref = m_run == kNegInf ? 0.f : m_run;  // keeps exp2(-inf - -inf) out of the picture
 
         float rs = 0.f;
         u32x4 pb[2][2];
@@ -308,51 +368,55 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
                 pb[kb][c] = u32x4{E::pack2(pf[0], pf[1]), E::pack2(pf[2], pf[3]), E::pack2(pf[4], pf[5]),
                                   E::pack2(pf[6], pf[7])};
             }
-        l_run = l_run * alpha + rs;
+        l_run += rs;
 
-#pragma unroll
-        for (int db = 0; db < D / 32; db++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) acc[db][i] *= alpha;
-
-        // O^T += V^T . P^T.  Transposing read: within each 16-lane group, lane t supplies the address of
-        // 4 consecutive d of key row (t>>2) and receives the 4 key rows of d column t.
-        const int tr_row = 4 * hh + ((lane & 15) >> 2);
-        const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+        // O^T += V^T . P^T
 #pragma unroll
         for (int db = 0; db < D / 32; db++)
 #pragma unroll
             for (int kc = 0; kc < 4; kc++) {
-                const uint8_t *vp = vb_ + (16 * kc + tr_row) * VSTR + (32 * db + tr_col) * 2;
+                const uint8_t *vp = vb_ + 16 * kc * ROWB + voff[db];
                 const u32x2 lo = E::tr_read(vp);
-                const u32x2 hi = E::tr_read(vp + 8 * VSTR);
+                const u32x2 hi = E::tr_read(vp + 8 * ROWB);
                 acc[db] = E::mfma(u32x4{lo.x, lo.y, hi.x, hi.y}, pb[kc >> 1][kc & 1], acc[db]);
             }
     };
 
     if (T > 0) {
-        int col_cur[EPC], col_nxt[EPC];
-        unsigned valid_cur, part_cur, valid_nxt = 0u, part_nxt = 0u;
-        u32x4 gk[NL], gv[NL];
-        chunk_entries(0, col_cur, valid_cur, part_cur);
-        load_chunk(col_cur, valid_cur, gk, gv);
-        store_chunk(0, gk, gv);
+        int col[EPC];
+        unsigned valid, part;
+        uint32_t mk_a[2][4] = {}, mk_b[2][4] = {};
+        bool sp_a, sp_b = false;
+        constexpr unsigned ALL = (1u << EPC) - 1u;
+        __syncthreads();  // the list in LDS is complete
+        chunk_entries(0, col, valid, part);
+        stage_chunk(0, col);
+        sp_a = part != 0u || valid != ALL;
+        if (sp_a) load_mask(col, valid, mk_a);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        for (int t = 0; t < T; t++) {
-            const bool more = t + 1 < T;
-            if (more) {
-                chunk_entries(t + 1, col_nxt, valid_nxt, part_nxt);
-                load_chunk(col_nxt, valid_nxt, gk, gv);
+        // Two chunks per trip so that the LDS buffer index is a compile-time constant.
+        for (int t = 0; t < T; t += 2) {
+            if (t + 1 < T) {
+                chunk_entries(t + 1, col, valid, part);
+                stage_chunk(1, col);
+                sp_b = part != 0u || valid != ALL;
+                if (sp_b) load_mask(col, valid, mk_b);
             }
-            compute(t & 1, col_cur, valid_cur, part_cur);
-            if (more) {
-                store_chunk((t + 1) & 1, gk, gv);
-#pragma unroll
-                for (int j = 0; j < EPC; j++) col_cur[j] = col_nxt[j];
-                valid_cur = valid_nxt;
-                part_cur = part_nxt;
-            }
+            compute(std::integral_constant<int, 0>{}, sp_a, mk_a);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
+            if (t + 1 < T) {
+                if (t + 2 < T) {
+                    chunk_entries(t + 2, col, valid, part);
+                    stage_chunk(0, col);
+                    sp_a = part != 0u || valid != ALL;
+                    if (sp_a) load_mask(col, valid, mk_a);
+                }
+                compute(std::integral_constant<int, 1>{}, sp_b, mk_b);
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+            }
         }
     }
 
@@ -372,7 +436,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
 
 template <int DT, int D, int NW, int MODE>
 hipError_t launch_one(const FwdParams &p, hipStream_t stream) {
-    constexpr int smem = 2 * 64 * (D * 2 + 16) + 2 * 64 * (D * 2 + 64);
+    constexpr int smem = 4 * 64 * D * 2 + kListCap * 4;  // two K and two V buffers of 64 rows + the list
     auto kern = sparse_fwd_kernel<DT, D, NW, MODE>;
     static bool attr_set = false;  // benign race: every thread sets the same value
     if (!attr_set) {
