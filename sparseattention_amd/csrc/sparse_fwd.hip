@@ -95,6 +95,22 @@ __device__ __forceinline__ float half_swap_sum(float x) {
 
 constexpr float kNegInf = -__builtin_inff();
 
+// 16 bytes per lane from global memory straight into LDS: lane i of the wave writes lds_base + 16*i.
+// Issued through inline assembly on purpose: the compiler then does not track it, so it does not hold
+// back later LDS reads of the OTHER buffer until the transfer lands.  Whoever reads the destination
+// must execute "s_waitcnt vmcnt(0)" and a workgroup barrier first (the main loop does).
+__device__ __forceinline__ void dma16(const void *gptr, const uint8_t *lds_base) {
+    const uint32_t lds_addr =
+        __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const SA_LDS uint8_t *)lds_base);
+    asm volatile(
+        "s_mov_b32 m0, %1\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %0, off"
+        :
+        : "v"(gptr), "s"(lds_addr)
+        : "memory");  // m0 is written; nothing else in these kernels keeps a value in it
+}
+
 // Swizzles of the 16-byte pieces inside an LDS row.  Rows are stored unpadded (D*2 bytes) because a
 // direct global->LDS load writes 64 lanes x 16 bytes contiguously; instead the piece index is XORed
 // with a function of the row so that
@@ -256,19 +272,17 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
             const int64_t srow = c0 + within;
             const uint16_t *gk = kbase + srow * p.ks[2] + 8 * (ld_slot ^ k_swizzle<D>(r));
             const uint16_t *gv = vbase + srow * p.vs[2] + 8 * (ld_slot ^ v_swizzle<D>(r));
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gk,
-                                             (SA_LDS void *)(smem + buf * KBUF + rbase * ROWB), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gv,
-                                             (SA_LDS void *)(smem + 2 * KBUF + buf * VBUF + rbase * ROWB), 16, 0, 0);
+            dma16(gk, smem + buf * KBUF + rbase * ROWB);
+            dma16(gv, smem + 2 * KBUF + buf * VBUF + rbase * ROWB);
         }
     };
 
     // Mask bytes of this lane's eight 4-key groups in a chunk (non-zero byte = attended key).  Called for
-    // chunks with a PARTIAL or absent entry only.  FULL entries are read too (their bytes are all set),
-    // absent entries are forced to zero: no branches, eight independent loads.
-    auto load_mask = [&](const int(&col)[EPC], unsigned valid, uint32_t(&mk)[2][4]) {
+    // chunks with a PARTIAL or absent entry only.  FULL entries are read too (their bytes are all set);
+    // absent entries re-read the chunk's first entry and are discarded when the mask is applied.
+    // No branches, eight independent loads, and no use of the loaded values here.
+    auto load_mask = [&](const int(&col)[EPC], uint32_t(&mk)[2][4]) {
         int64_t c[2][4];
-        uint32_t keep[2][4];
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
@@ -285,51 +299,62 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
                     within = 32 * kb + 8 * g + 4 * hh;
                 }
                 c[kb][g] = col[j] + within;
-                keep[kb][g] = ((valid >> j) & 1u) ? 0xffffffffu : 0u;
             }
         if (p.mask_vec4) {
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-                for (int g = 0; g < 4; g++) mk[kb][g] = *(const uint32_t *)(mrow + c[kb][g]) & keep[kb][g];
+                for (int g = 0; g < 4; g++) mk[kb][g] = *(const uint32_t *)(mrow + c[kb][g]);
         } else {
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
                     const uint8_t *m0 = mrow + c[kb][g] * p.ms[3];
-                    mk[kb][g] = ((uint32_t)m0[0] | ((uint32_t)m0[p.ms[3]] << 8) | ((uint32_t)m0[2 * p.ms[3]] << 16) |
-                                 ((uint32_t)m0[3 * p.ms[3]] << 24)) & keep[kb][g];
+                    mk[kb][g] = (uint32_t)m0[0] | ((uint32_t)m0[p.ms[3]] << 8) | ((uint32_t)m0[2 * p.ms[3]] << 16) |
+                                ((uint32_t)m0[3 * p.ms[3]] << 24);
                 }
         }
     };
 
-    auto compute = [&](auto buf_c, bool special, const uint32_t(&mk)[2][4]) {
+    auto compute = [&](auto buf_c, bool special, unsigned valid, const uint32_t(&mk)[2][4]) {
         constexpr int BUF = decltype(buf_c)::value;
         const uint8_t *kb_ = smem + BUF * KBUF;
         const uint8_t *vb_ = smem + 2 * KBUF + BUF * VBUF;
 
-        // S^T = K . Q^T
+        // S^T = K . Q^T: MFMA i works on d step i/2 of key block i%2.  All operand reads are written
+        // first and the scheduling groups below interleave them: kPfS reads in flight ahead of the MFMAs.
+        constexpr int NS = 2 * (D / 16);
+        constexpr int kPfS = 6;
         f32x16 s[2];
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
+        for (int kb = 0; kb < 2; kb++)
 #pragma unroll
             for (int i = 0; i < 16; i++) s[kb][i] = 0.f;
+        u32x4 kfr[NS];
 #pragma unroll
-            for (int c = 0; c < D / 16; c++) {
-                const u32x4 a = *(const u32x4 *)(kb_ + 32 * kb * ROWB + koff[c]);
-                s[kb] = E::mfma(a, qf[c], s[kb]);
-            }
+        for (int i = 0; i < NS; i++) kfr[i] = *(const u32x4 *)(kb_ + 32 * (i & 1) * ROWB + koff[i >> 1]);
+#pragma unroll
+        for (int i = 0; i < NS; i++) s[i & 1] = E::mfma(kfr[i], qf[i >> 1], s[i & 1]);
+        __builtin_amdgcn_sched_group_barrier(0x100, kPfS, 0);
+#pragma unroll
+        for (int i = 0; i < NS - kPfS; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
+        __builtin_amdgcn_sched_group_barrier(0x008, kPfS, 0);
 
         if (special) {
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-                for (int g = 0; g < 4; g++)
+                for (int g = 0; g < 4; g++) {
+                    const int j = MODE == 0 ? 2 * kb + (g >> 1) : (MODE == 1 ? kb : 0);  // list entry of this group
+                    const uint32_t w = ((valid >> j) & 1u) ? mk[kb][g] : 0u;
 #pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        if (((mk[kb][g] >> (8 * j)) & 0xffu) == 0u) s[kb][4 * g + j] = kNegInf;
+                    for (int jj = 0; jj < 4; jj++)
+                        if (((w >> (8 * jj)) & 0xffu) == 0u) s[kb][4 * g + jj] = kNegInf;
+                }
         }
 
         // Online softmax in exp2 units (sparse_attn_kernel.py:47-58), with a lagging reference value.
@@ -353,38 +378,67 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         }
         const float m_ref = m_run == kNegInf ? 0.f : m_run;  // keeps exp2(-inf - -inf) out of the picture
 
+        // P = exp2(S*scale - m_ref), rounded to the input dtype, and O^T += V^T . P^T.
+        // MFMA i = (key step kc = i / NDB, d block db = i % NDB) needs only the kc-th group of 8 P values, so
+        // the loop is written as a software pipeline of bundles, each pinned by a scheduling barrier:
+        //   one MFMA | the transposing reads of the operand kPfV MFMAs ahead | a share of the next
+        //   group's exponentials.
+        constexpr int NDB = D / 32;
+        constexpr int NV = 4 * NDB;
+        constexpr int kPfV = 3;
+        constexpr int PER = 8 / NDB;  // P values of the next group produced per bundle
         float rs = 0.f;
-        u32x4 pb[2][2];
+        float pf[4][8];
+        u32x4 pb[4];
+        u32x2 vlo[NV], vhi[NV];
+        auto p_values = [&](int kc, int first, int count) {
+#pragma unroll
+            for (int i = first; i < first + count; i++) {
+                pf[kc][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kc >> 1][8 * (kc & 1) + i], p.scale, -m_ref));
+                rs += pf[kc][i];
+            }
+        };
+        auto p_pack = [&](int kc) {
+            pb[kc] = u32x4{E::pack2(pf[kc][0], pf[kc][1]), E::pack2(pf[kc][2], pf[kc][3]), E::pack2(pf[kc][4], pf[kc][5]),
+                           E::pack2(pf[kc][6], pf[kc][7])};
+        };
+        auto v_read = [&](int i) {
+            const uint8_t *vp = vb_ + 16 * (i / NDB) * ROWB + voff[i % NDB];
+            vlo[i] = E::tr_read(vp);
+            vhi[i] = E::tr_read(vp + 8 * ROWB);
+        };
+#pragma unroll
+        for (int i = 0; i < kPfV; i++) v_read(i);
+        p_values(0, 0, 8);
+        p_pack(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int kc = i / NDB, db = i % NDB;
+            acc[db] = E::mfma(u32x4{vlo[i].x, vlo[i].y, vhi[i].x, vhi[i].y}, pb[kc], acc[db]);
+            if (i + kPfV < NV) v_read(i + kPfV);
+            if (kc + 1 < 4) {
+                p_values(kc + 1, PER * db, PER);
+                if (db == NDB - 1) p_pack(kc + 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        l_run += rs;
+    };
+
+    // Makes the compiler account for a completed vector-memory load here (it emits its own wait, which
+    // costs nothing once the data has landed) instead of in front of a later use, where the wait would
+    // also cover direct loads it does not know about.
+    auto settle = [](const uint32_t(&mk)[2][4]) {
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-            for (int c = 0; c < 2; c++) {
-                float pf[8];
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    pf[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][8 * c + i], p.scale, -m_ref));
-                    rs += pf[i];
-                }
-                pb[kb][c] = u32x4{E::pack2(pf[0], pf[1]), E::pack2(pf[2], pf[3]), E::pack2(pf[4], pf[5]),
-                                  E::pack2(pf[6], pf[7])};
-            }
-        l_run += rs;
-
-        // O^T += V^T . P^T
-#pragma unroll
-        for (int db = 0; db < D / 32; db++)
-#pragma unroll
-            for (int kc = 0; kc < 4; kc++) {
-                const uint8_t *vp = vb_ + 16 * kc * ROWB + voff[db];
-                const u32x2 lo = E::tr_read(vp);
-                const u32x2 hi = E::tr_read(vp + 8 * ROWB);
-                acc[db] = E::mfma(u32x4{lo.x, lo.y, hi.x, hi.y}, pb[kc >> 1][kc & 1], acc[db]);
-            }
+            for (int g = 0; g < 4; g++) asm volatile("" ::"v"(mk[kb][g]));
     };
 
     if (T > 0) {
         int col[EPC];
-        unsigned valid, part;
+        unsigned valid, part, valid_a, valid_b = 0u;
         uint32_t mk_a[2][4] = {}, mk_b[2][4] = {};
         bool sp_a, sp_b = false;
         constexpr unsigned ALL = (1u << EPC) - 1u;
@@ -392,7 +446,11 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         chunk_entries(0, col, valid, part);
         stage_chunk(0, col);
         sp_a = part != 0u || valid != ALL;
-        if (sp_a) load_mask(col, valid, mk_a);
+        valid_a = valid;
+        if (sp_a) load_mask(col, mk_a);
+#pragma unroll
+        for (int c = 0; c < D / 16; c++) asm volatile("" ::"v"(qf[c]));
+        settle(mk_a);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         // Two chunks per trip so that the LDS buffer index is a compile-time constant.
@@ -401,20 +459,24 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
                 chunk_entries(t + 1, col, valid, part);
                 stage_chunk(1, col);
                 sp_b = part != 0u || valid != ALL;
-                if (sp_b) load_mask(col, valid, mk_b);
+                valid_b = valid;
+                if (sp_b) load_mask(col, mk_b);
             }
-            compute(std::integral_constant<int, 0>{}, sp_a, mk_a);
+            compute(std::integral_constant<int, 0>{}, sp_a, valid_a, mk_a);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            settle(mk_b);
             __syncthreads();
             if (t + 1 < T) {
                 if (t + 2 < T) {
                     chunk_entries(t + 2, col, valid, part);
                     stage_chunk(0, col);
                     sp_a = part != 0u || valid != ALL;
-                    if (sp_a) load_mask(col, valid, mk_a);
+                    valid_a = valid;
+                    if (sp_a) load_mask(col, mk_a);
                 }
-                compute(std::integral_constant<int, 1>{}, sp_b, mk_b);
+                compute(std::integral_constant<int, 1>{}, sp_b, valid_b, mk_b);
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                settle(mk_a);
                 __syncthreads();
             }
         }
