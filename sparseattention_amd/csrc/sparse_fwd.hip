@@ -95,19 +95,24 @@ __device__ __forceinline__ float half_swap_sum(float x) {
 
 constexpr float kNegInf = -__builtin_inff();
 
-// 16 bytes per lane from global memory straight into LDS: lane i of the wave writes lds_base + 16*i.
+// 16 bytes per lane from global memory (wave-uniform base + per-lane byte offset) straight into LDS:
+// lane i of the wave writes LDS address lds_addr + 16*i.
 // Issued through inline assembly on purpose: the compiler then does not track it, so it does not hold
 // back later LDS reads of the OTHER buffer until the transfer lands.  Whoever reads the destination
 // must execute "s_waitcnt vmcnt(0)" and a workgroup barrier first (the main loop does).
-__device__ __forceinline__ void dma16(const void *gptr, const uint8_t *lds_base) {
-    const uint32_t lds_addr =
-        __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const SA_LDS uint8_t *)lds_base);
+__device__ __forceinline__ void dma16(const void *base, uint32_t lane_offset, uint32_t lds_addr) {
+    // the base is wave-uniform by construction; say so in a way the register allocator cannot miss
+    const uint64_t b = (uint64_t)(uintptr_t)base;
+    // (readfirstlane returns a signed int: widen through uint32_t, or the low half sign-extends)
+    const uint64_t ub = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b) |
+                        ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32)) << 32);
+    lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
     asm volatile(
-        "s_mov_b32 m0, %1\n\t"
+        "s_mov_b32 m0, %2\n\t"
         "s_nop 0\n\t"
-        "global_load_lds_dwordx4 %0, off"
+        "global_load_lds_dwordx4 %0, %1"
         :
-        : "v"(gptr), "s"(lds_addr)
+        : "v"(lane_offset), "s"(ub), "s"(lds_addr)
         : "memory");  // m0 is written; nothing else in these kernels keeps a value in it
 }
 
@@ -212,7 +217,20 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
     }
     // Direct-load staging: load i of this wave fills rows [RPI*(NW*i + wave), +RPI) of the chunk; lane
     // writes row ld_row(i), LDS piece lane % PPR, and therefore fetches the swizzled source piece.
+    // The source address splits into a wave-uniform part (plane base + first row of the list entry, scalar
+    // arithmetic per chunk) and a per-lane byte offset that never changes (row within the entry, swizzled
+    // piece), so staging a chunk costs no vector arithmetic.
     const int ld_r0 = lane / PPR, ld_slot = lane % PPR;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const SA_LDS uint8_t *)smem);
+    uint32_t ld_koff[NLD], ld_voff[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; i++) {
+        const int r = RPI * (NW * i + wave_u) + ld_r0;
+        const int within = MODE == 2 ? r : (r & ((1 << LBKC) - 1));
+        ld_koff[i] = (uint32_t)((within * p.ks[2] + 8 * (ld_slot ^ k_swizzle<D>(r))) * 2);
+        ld_voff[i] = (uint32_t)((within * p.vs[2] + 8 * (ld_slot ^ v_swizzle<D>(r))) * 2);
+    }
 
     // The Q tile's list (FULL entries, then PARTIAL entries) as first key columns, copied to LDS once:
     // loads issued after the first barrier cannot use the scalar cache, and a vector load of an index in
@@ -224,10 +242,15 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
             ent[e] = MODE == 2 ? (idx << p.lbk) : (idx << LBKC);
         }
     }
-    auto entry_col = [&](int e) -> int {
-        if (list_in_lds) return ent[e];
-        const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
-        return MODE == 2 ? (idx << p.lbk) : (idx << LBKC);
+    auto entry_col = [&](int e) -> int {  // wave-uniform result, kept in a scalar register
+        int c;
+        if (list_in_lds) {
+            c = ent[e];
+        } else {
+            const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
+            c = MODE == 2 ? (idx << p.lbk) : (idx << LBKC);
+        }
+        return __builtin_amdgcn_readfirstlane(c);
     };
 
     // First key column of every list entry in chunk t (t < T), plus which entries exist / are partial.
@@ -258,22 +281,15 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
     auto stage_chunk = [&](int buf, const int(&col)[EPC]) {
 #pragma unroll
         for (int i = 0; i < NLD; i++) {
-            const int rbase = RPI * (NW * i + wave);  // wave-uniform
-            const int r = rbase + ld_r0;
-            int j = 0, within = r;
-            if constexpr (MODE != 2) {
-                j = r >> LBKC;
-                within = r & ((1 << LBKC) - 1);
-            }
+            const int rbase = RPI * (NW * i + wave_u);  // rows [rbase, rbase + RPI) lie inside one list entry
             int c0 = col[0];
+            if constexpr (MODE != 2) {
 #pragma unroll
-            for (int jj = 1; jj < EPC; jj++)
-                if (j == jj) c0 = col[jj];
-            const int64_t srow = c0 + within;
-            const uint16_t *gk = kbase + srow * p.ks[2] + 8 * (ld_slot ^ k_swizzle<D>(r));
-            const uint16_t *gv = vbase + srow * p.vs[2] + 8 * (ld_slot ^ v_swizzle<D>(r));
-            dma16(gk, smem + buf * KBUF + rbase * ROWB);
-            dma16(gv, smem + 2 * KBUF + buf * VBUF + rbase * ROWB);
+                for (int jj = 1; jj < EPC; jj++)
+                    if ((rbase >> LBKC) == jj) c0 = col[jj];
+            }
+            dma16(kbase + (int64_t)c0 * p.ks[2], ld_koff[i], lds0 + buf * KBUF + rbase * ROWB);
+            dma16(vbase + (int64_t)c0 * p.vs[2], ld_voff[i], lds0 + 2 * KBUF + buf * VBUF + rbase * ROWB);
         }
     };
 
