@@ -63,6 +63,11 @@ struct Elem<0> {  // bf16
     static __device__ __forceinline__ u32x2 tr_read(const uint8_t *lds_ptr) {
         return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((SA_LDS bf16x4 *)lds_ptr));
     }
+    // c + lo + hi of a packed pair, accumulated in fp32 (one instruction instead of two additions)
+    static __device__ __forceinline__ float add_pair(uint32_t pk, float c) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk), __builtin_bit_cast(bf16x2, 0x3f803f80u), c,
+                                               false);
+    }
 };
 
 template <>
@@ -78,6 +83,9 @@ struct Elem<1> {  // fp16
     static __device__ __forceinline__ u32x2 tr_read(const uint8_t *lds_ptr) {
         // the transposing read only moves 16-bit lanes around, so the bf16 flavour serves fp16 too
         return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((SA_LDS bf16x4 *)lds_ptr));
+    }
+    static __device__ __forceinline__ float add_pair(uint32_t pk, float c) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pk), __builtin_bit_cast(f16x2, 0x3c003c00u), c, false);
     }
 };
 
@@ -279,17 +287,30 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
 
     // Global -> LDS for one chunk, without passing through registers.
     auto stage_chunk = [&](int buf, const int(&col)[EPC]) {
+        const uint16_t *kp[EPC], *vp[EPC];  // first row of every list entry of the chunk (scalar registers)
+#pragma unroll
+        for (int j = 0; j < EPC; j++) {
+            kp[j] = kbase + (int64_t)col[j] * p.ks[2];
+            vp[j] = vbase + (int64_t)col[j] * p.vs[2];
+        }
 #pragma unroll
         for (int i = 0; i < NLD; i++) {
-            const int rbase = RPI * (NW * i + wave_u);  // rows [rbase, rbase + RPI) lie inside one list entry
-            int c0 = col[0];
+            // rows [rbase, rbase + RPI) lie inside one list entry; when the rows of all waves of load i do,
+            // the entry is known at compile time
+            constexpr bool kEntryByLoad = MODE == 2 || RPI * NW <= (1 << LBKC);
+            const int rbase = RPI * (NW * i + wave_u);
+            const uint16_t *ks_ = kp[0], *vs_ = vp[0];
             if constexpr (MODE != 2) {
+                const int j = kEntryByLoad ? ((RPI * NW * i) >> LBKC) : (rbase >> LBKC);
 #pragma unroll
                 for (int jj = 1; jj < EPC; jj++)
-                    if ((rbase >> LBKC) == jj) c0 = col[jj];
+                    if (j == jj) {
+                        ks_ = kp[jj];
+                        vs_ = vp[jj];
+                    }
             }
-            dma16(kbase + (int64_t)c0 * p.ks[2], ld_koff[i], lds0 + buf * KBUF + rbase * ROWB);
-            dma16(vbase + (int64_t)c0 * p.vs[2], ld_voff[i], lds0 + 2 * KBUF + buf * VBUF + rbase * ROWB);
+            dma16(ks_, ld_koff[i], lds0 + buf * KBUF + rbase * ROWB);
+            dma16(vs_, ld_voff[i], lds0 + 2 * KBUF + buf * VBUF + rbase * ROWB);
         }
     };
 
@@ -403,21 +424,23 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         constexpr int NV = 4 * NDB;
         constexpr int kPfV = 3;
         constexpr int PER = 8 / NDB;  // P values of the next group produced per bundle
-        float rs = 0.f;
-        float pf[4][8];
-        u32x4 pb[4];
-        u32x2 vlo[NV], vhi[NV];
+        // The row sum adds up the ROUNDED values, the ones that enter P.V, so the output is an exact convex
+        // combination of value rows (the reference sums the unrounded ones; the difference is bounded by the
+        // rounding of P itself).
+        float rs0 = 0.f, rs1 = 0.f;
+        uint32_t pw[16];  // P, two keys per dword, in MFMA operand order
         auto p_values = [&](int kc, int first, int count) {
 #pragma unroll
-            for (int i = first; i < first + count; i++) {
-                pf[kc][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kc >> 1][8 * (kc & 1) + i], p.scale, -m_ref));
-                rs += pf[kc][i];
+            for (int i = first; i < first + count; i += 2) {
+                const float x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kc >> 1][8 * (kc & 1) + i], p.scale, -m_ref));
+                const float x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kc >> 1][8 * (kc & 1) + i + 1], p.scale, -m_ref));
+                const uint32_t w = E::pack2(x0, x1);
+                pw[4 * kc + (i >> 1)] = w;
+                if (i & 2) rs1 = E::add_pair(w, rs1);
+                else rs0 = E::add_pair(w, rs0);
             }
         };
-        auto p_pack = [&](int kc) {
-            pb[kc] = u32x4{E::pack2(pf[kc][0], pf[kc][1]), E::pack2(pf[kc][2], pf[kc][3]), E::pack2(pf[kc][4], pf[kc][5]),
-                           E::pack2(pf[kc][6], pf[kc][7])};
-        };
+        u32x2 vlo[NV], vhi[NV];
         auto v_read = [&](int i) {
             const uint8_t *vp = vb_ + 16 * (i / NDB) * ROWB + voff[i % NDB];
             vlo[i] = E::tr_read(vp);
@@ -426,20 +449,17 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
 #pragma unroll
         for (int i = 0; i < kPfV; i++) v_read(i);
         p_values(0, 0, 8);
-        p_pack(0);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < NV; i++) {
             const int kc = i / NDB, db = i % NDB;
-            acc[db] = E::mfma(u32x4{vlo[i].x, vlo[i].y, vhi[i].x, vhi[i].y}, pb[kc], acc[db]);
+            acc[db] = E::mfma(u32x4{vlo[i].x, vlo[i].y, vhi[i].x, vhi[i].y},
+                              u32x4{pw[4 * kc], pw[4 * kc + 1], pw[4 * kc + 2], pw[4 * kc + 3]}, acc[db]);
             if (i + kPfV < NV) v_read(i + kPfV);
-            if (kc + 1 < 4) {
-                p_values(kc + 1, PER * db, PER);
-                if (db == NDB - 1) p_pack(kc + 1);
-            }
+            if (kc + 1 < 4) p_values(kc + 1, PER * db, PER);
             __builtin_amdgcn_sched_barrier(0);
         }
-        l_run += rs;
+        l_run += rs0 + rs1;
     };
 
     // Makes the compiler account for a completed vector-memory load here (it emits its own wait, which
