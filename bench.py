@@ -29,6 +29,12 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak, TFLOP/s
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E peak, GB/s
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this script and scaled by
+# the readings of a 1 GiB device copy in the same run (--calibrate-copy).  The summaries with the commands
+# are profiles/sparse_fwd_kernel_causal_B8H32S4096D128.txt and profiles/mask_classify_kernels_mask_32768x32768.txt.
+TRAFFIC_FWD_CAUSAL_BYTES = 1.2284e9      # 915.4 MiB read + 256.1 MiB written
+TRAFFIC_CLASSIFY_1GIB_BYTES = 1.0745e9   # 1,048,648 + 331 KiB read, 256 + 45.5 KiB written
+
 B, H, S, D = 8, 32, 4096, 128
 BQ, BK = 128, 32
 FLOP_PER_TILE = 4 * BQ * BK * D
@@ -42,6 +48,9 @@ def parse():
     ap.add_argument("--no-sweep", action="store_true", help="skip the across-p table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--no-classify", action="store_true", help="skip the mask-classification timing")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy a few times, so that a counter run over this command "
+                         "holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     return ap.parse_args()
 
 
@@ -123,7 +132,8 @@ def classify_case(steps, warmup):
         "workload": "sa_mask_classify on the composed mask, bool [32768,32768] = 1 GiB, tiles 128x32",
         "ms": round(ev_ms, 4),
         "roofline": {"bound": "hbm", "achieved": round(nbytes / (ev_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(nbytes / (ev_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None},
+                     "unit": "GB/s", "frac": round(nbytes / (ev_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                     "traffic": TRAFFIC_CLASSIFY_1GIB_BYTES, "algorithmic_bytes": nbytes},
     }
 
 
@@ -224,7 +234,7 @@ def main():
                    "executed_tiles_per_plane": int(head["_executed_flop"] // (B * H * FLOP_PER_TILE)),
                    "partial_tiles_per_plane": head["partial_tiles_per_plane"]},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_FWD_CAUSAL_BYTES,
                      "kernel": "sparse_fwd_kernel", "kernel_ms": head["kernel_ms"],
                      "flop_per_launch": head["_executed_flop"]},
     }
@@ -241,6 +251,13 @@ def main():
         result["mask_classify"] = classify_case(max(10, args.steps // 2), max(3, args.warmup // 2))
         result["mask_classify_headline"] = classify_small_case(max(10, args.steps // 2), max(3, args.warmup // 2))
     del q, k, v
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, dtype=torch.int32, device="cuda")  # 1 GiB read + 1 GiB written per copy
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if not args.no_cpu:
         result.update(cpu_baselines())
     print(json.dumps(result))
