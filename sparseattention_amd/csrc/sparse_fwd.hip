@@ -63,10 +63,8 @@ struct Elem<0> {  // bf16
     static __device__ __forceinline__ u32x2 tr_read(const uint8_t *lds_ptr) {
         return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((SA_LDS bf16x4 *)lds_ptr));
     }
-    // c + lo + hi of a packed pair, accumulated in fp32 (one instruction instead of two additions)
-    static __device__ __forceinline__ float add_pair(uint32_t pk, float c) {
-        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk), __builtin_bit_cast(bf16x2, 0x3f803f80u), c,
-                                               false);
+    static __device__ __forceinline__ u32x4 ones4() {  // eight 1.0 values, an all-ones MFMA operand
+        return u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
     }
 };
 
@@ -84,8 +82,8 @@ struct Elem<1> {  // fp16
         // the transposing read only moves 16-bit lanes around, so the bf16 flavour serves fp16 too
         return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((SA_LDS bf16x4 *)lds_ptr));
     }
-    static __device__ __forceinline__ float add_pair(uint32_t pk, float c) {
-        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pk), __builtin_bit_cast(f16x2, 0x3c003c00u), c, false);
+    static __device__ __forceinline__ u32x4 ones4() {
+        return u32x4{0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};
     }
 };
 
@@ -94,11 +92,6 @@ __device__ __forceinline__ float half_swap_max(float x) {
     const uint32_t u = __float_as_uint(x);
     const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
     return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float half_swap_sum(float x) {
-    const uint32_t u = __float_as_uint(x);
-    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
 constexpr float kNegInf = -__builtin_inff();
@@ -198,7 +191,9 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
     }
 
     float m_run = kNegInf;  // reference value of the row's exponentials, in exp2 units (score * scale)
-    float l_run = 0.f;      // running row sum over this lane's half of the keys
+    f32x16 acc_l;           // every element: running row sum of P for this lane's query (see the P.V loop)
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc_l[i] = 0.f;
     f32x16 acc[D / 32];
 #pragma unroll
     for (int db = 0; db < D / 32; db++)
@@ -359,27 +354,30 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         const uint8_t *kb_ = smem + BUF * KBUF;
         const uint8_t *vb_ = smem + 2 * KBUF + BUF * VBUF;
 
-        // S^T = K . Q^T: MFMA i works on d step i/2 of key block i%2.  All operand reads are written
-        // first and the scheduling groups below interleave them: kPfS reads in flight ahead of the MFMAs.
-        constexpr int NS = 2 * (D / 16);
-        constexpr int kPfS = 6;
+        // S^T = K . Q^T in bundles of two MFMAs (the two key blocks of d step c), operand reads kPfS bundles
+        // ahead.  Within a bundle the MFMA that uses the younger read goes first, so one wait covers both.
+        constexpr int NC = D / 16;
+        constexpr int kPfS = 3;
         f32x16 s[2];
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
             for (int i = 0; i < 16; i++) s[kb][i] = 0.f;
-        u32x4 kfr[NS];
+        u32x4 kf0[NC], kf1[NC];
+        auto k_read = [&](int c) {
+            kf0[c] = *(const u32x4 *)(kb_ + koff[c]);
+            kf1[c] = *(const u32x4 *)(kb_ + 32 * ROWB + koff[c]);
+        };
 #pragma unroll
-        for (int i = 0; i < NS; i++) kfr[i] = *(const u32x4 *)(kb_ + 32 * (i & 1) * ROWB + koff[i >> 1]);
+        for (int c = 0; c < kPfS; c++) k_read(c);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < NS; i++) s[i & 1] = E::mfma(kfr[i], qf[i >> 1], s[i & 1]);
-        __builtin_amdgcn_sched_group_barrier(0x100, kPfS, 0);
-#pragma unroll
-        for (int i = 0; i < NS - kPfS; i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        for (int c = 0; c < NC; c++) {
+            s[1] = E::mfma(kf1[c], qf[c], s[1]);
+            s[0] = E::mfma(kf0[c], qf[c], s[0]);
+            if (c + kPfS < NC) k_read(c + kPfS);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, kPfS, 0);
 
         if (special) {
 #pragma unroll
@@ -407,7 +405,8 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
             const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // m_new is finite wherever raise holds
             const float a = raise ? alpha : 1.f;
             m_run = m_new;
-            l_run *= a;
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc_l[i] *= a;
 #pragma unroll
             for (int db = 0; db < D / 32; db++)
 #pragma unroll
@@ -416,50 +415,55 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         const float m_ref = m_run == kNegInf ? 0.f : m_run;  // keeps exp2(-inf - -inf) out of the picture
 
         // P = exp2(S*scale - m_ref), rounded to the input dtype, and O^T += V^T . P^T.
-        // MFMA i = (key step kc = i / NDB, d block db = i % NDB) needs only the kc-th group of 8 P values, so
-        // the loop is written as a software pipeline of bundles, each pinned by a scheduling barrier:
-        //   one MFMA | the transposing reads of the operand kPfV MFMAs ahead | a share of the next
-        //   group's exponentials.
+        // MFMA (key step kc, d block db) needs only the kc-th group of 8 P values, so the loop is a software
+        // pipeline of bundles pinned by scheduling barriers: two MFMAs (d blocks 2h, 2h+1 of one key step) |
+        // the transposing reads for a later bundle | half of the next key step's exponentials.
+        // The row sum comes from one more MFMA per key step whose A operand is all ones: every row of its
+        // result is sum_k P[k][q] over the 16 keys of the step, both lane halves included.  It therefore adds
+        // up the ROUNDED values, the ones that enter P.V, and the output is an exact convex combination of
+        // value rows (the reference sums the unrounded ones; the difference is bounded by the rounding of P).
         constexpr int NDB = D / 32;
-        constexpr int NV = 4 * NDB;
-        constexpr int kPfV = 3;
-        constexpr int PER = 8 / NDB;  // P values of the next group produced per bundle
-        // The row sum adds up the ROUNDED values, the ones that enter P.V, so the output is an exact convex
-        // combination of value rows (the reference sums the unrounded ones; the difference is bounded by the
-        // rounding of P itself).
-        float rs0 = 0.f, rs1 = 0.f;
-        uint32_t pw[16];  // P, two keys per dword, in MFMA operand order
+        constexpr int NB = 4 * NDB / 2;  // bundles; bundle b: key step b / (NDB/2), d blocks 2*(b % (NDB/2)) + {0,1}
+        constexpr int BPK = NDB / 2;     // bundles per key step
+        constexpr int kPfV = 2;
+        constexpr int PER = 8 / BPK;     // P values of the next key step produced per bundle
+        uint32_t pw[16];                 // P, two keys per dword, in MFMA operand order
         auto p_values = [&](int kc, int first, int count) {
 #pragma unroll
             for (int i = first; i < first + count; i += 2) {
                 const float x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kc >> 1][8 * (kc & 1) + i], p.scale, -m_ref));
                 const float x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kc >> 1][8 * (kc & 1) + i + 1], p.scale, -m_ref));
-                const uint32_t w = E::pack2(x0, x1);
-                pw[4 * kc + (i >> 1)] = w;
-                if (i & 2) rs1 = E::add_pair(w, rs1);
-                else rs0 = E::add_pair(w, rs0);
+                pw[4 * kc + (i >> 1)] = E::pack2(x0, x1);
             }
         };
-        u32x2 vlo[NV], vhi[NV];
-        auto v_read = [&](int i) {
-            const uint8_t *vp = vb_ + 16 * (i / NDB) * ROWB + voff[i % NDB];
-            vlo[i] = E::tr_read(vp);
-            vhi[i] = E::tr_read(vp + 8 * ROWB);
+        u32x2 vlo[2 * NB], vhi[2 * NB];
+        auto v_read = [&](int b) {
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                const int kc = b / BPK, db = 2 * (b % BPK) + u;
+                const uint8_t *vp = vb_ + 16 * kc * ROWB + voff[db];
+                vlo[2 * b + u] = E::tr_read(vp);
+                vhi[2 * b + u] = E::tr_read(vp + 8 * ROWB);
+            }
         };
 #pragma unroll
-        for (int i = 0; i < kPfV; i++) v_read(i);
+        for (int b = 0; b < kPfV; b++) v_read(b);
         p_values(0, 0, 8);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < NV; i++) {
-            const int kc = i / NDB, db = i % NDB;
-            acc[db] = E::mfma(u32x4{vlo[i].x, vlo[i].y, vhi[i].x, vhi[i].y},
-                              u32x4{pw[4 * kc], pw[4 * kc + 1], pw[4 * kc + 2], pw[4 * kc + 3]}, acc[db]);
-            if (i + kPfV < NV) v_read(i + kPfV);
-            if (kc + 1 < 4) p_values(kc + 1, PER * db, PER);
+        for (int b = 0; b < NB; b++) {
+            const int kc = b / BPK;
+            const u32x4 pk4 = u32x4{pw[4 * kc], pw[4 * kc + 1], pw[4 * kc + 2], pw[4 * kc + 3]};
+#pragma unroll
+            for (int u = 1; u >= 0; u--) {
+                const int db = 2 * (b % BPK) + u, i = 2 * b + u;
+                acc[db] = E::mfma(u32x4{vlo[i].x, vlo[i].y, vhi[i].x, vhi[i].y}, pk4, acc[db]);
+            }
+            if (b % BPK == BPK - 1) acc_l = E::mfma(E::ones4(), pk4, acc_l);
+            if (b + kPfV < NB) v_read(b + kPfV);
+            if (kc + 1 < 4) p_values(kc + 1, PER * (b % BPK), PER);
             __builtin_amdgcn_sched_barrier(0);
         }
-        l_run += rs0 + rs1;
     };
 
     // Makes the compiler account for a completed vector-memory load here (it emits its own wait, which
@@ -519,7 +523,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
     }
 
     // Epilogue: O = acc / l (sparse_attn_kernel.py:144); rows that attended to nothing give 0.
-    const float l_tot = half_swap_sum(l_run);
+    const float l_tot = acc_l[0];
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     uint16_t *orow = p.o + b * p.os[0] + h * p.os[1] + (int64_t)qrow * p.os[2] + 4 * hh;
 #pragma unroll
@@ -561,6 +565,7 @@ hipError_t launch_bq(const FwdParams &p, int BQ, hipStream_t stream) {
         case 32: return launch_mode<DT, D, 1>(p, stream);
         case 64: return launch_mode<DT, D, 2>(p, stream);
         case 128: return launch_mode<DT, D, 4>(p, stream);
+        case 256: return launch_mode<DT, D, 8>(p, stream);
         default: return hipErrorInvalidValue;
     }
 }

@@ -154,8 +154,8 @@ int sa_sparse_attention_fwd(const void *q, const int64_t q_strides[4], const voi
     if (dtype != SA_DTYPE_BF16 && dtype != SA_DTYPE_FP16)
         return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: dtype code %d (supported: 0 = bf16, 1 = fp16)", dtype);
     if (D != 64 && D != 128) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: head dim %d (supported: 64, 128)", D);
-    if (BQ != 32 && BQ != 64 && BQ != 128)
-        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: BLOCK_Q %d (supported: 32, 64, 128)", BQ);
+    if (BQ != 32 && BQ != 64 && BQ != 128 && BQ != 256)
+        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: BLOCK_Q %d (supported: 32, 64, 128, 256)", BQ);
     const int lbk = log2_exact(BK);
     if (lbk < 4) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: BLOCK_K %d (supported: powers of two >= 16)", BK);
     const int64_t *st[4] = {q_strides, k_strides, v_strides, o_strides};

@@ -90,6 +90,7 @@ def test_forward_rejects_bad_arguments():
     assert fwd(scale=float("nan")) == _native.SA_ERR_INVALID_ARGUMENT
     assert fwd(D=96) == _native.SA_ERR_UNSUPPORTED and "head dim" in last_error()
     assert fwd(BQ=16, Sq=256) == _native.SA_ERR_UNSUPPORTED and "BLOCK_Q" in last_error()
+    assert fwd(BQ=512, Sq=512) == _native.SA_ERR_UNSUPPORTED and "BLOCK_Q" in last_error()
     assert fwd(BK=8) == _native.SA_ERR_UNSUPPORTED and "BLOCK_K" in last_error()
     assert fwd(BK=4, Sk=252, Sq=256) == _native.SA_ERR_UNSUPPORTED
     assert fwd(dtype=7) == _native.SA_ERR_UNSUPPORTED and "dtype" in last_error()

@@ -32,7 +32,7 @@ def oracle_out(q, k, v, mask, BQ, BK, p_round):
 
 
 @pytest.mark.parametrize("D", [64, 128])
-@pytest.mark.parametrize("BQ", [32, 64, 128])
+@pytest.mark.parametrize("BQ", [32, 64, 128, 256])
 @pytest.mark.parametrize("BK", [16, 32, 64, 128, 256])
 def test_tile_shapes_against_oracle_and_sdpa(gpu, D, BQ, BK):
     B, H, S = 2, 2, 512
