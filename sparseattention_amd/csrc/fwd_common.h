@@ -1,0 +1,120 @@
+// Helpers shared by the forward kernels: register types, per-dtype MFMA wrappers, the direct global->LDS
+// load, the LDS row swizzles and the constants of the online softmax.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+#include "kernels.h"
+
+namespace sa {
+namespace {
+
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+#define SA_LDS __attribute__((address_space(3)))
+
+template <int DT>
+struct Elem;
+
+template <>
+struct Elem<0> {  // bf16
+    static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                       0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        const f32x2 f = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+    }
+    static __device__ __forceinline__ u32x2 tr_read(const uint8_t *lds_ptr) {
+        return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((SA_LDS bf16x4 *)lds_ptr));
+    }
+    static __device__ __forceinline__ u32x4 ones4() {  // eight 1.0 values, an all-ones MFMA operand
+        return u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+    }
+};
+
+template <>
+struct Elem<1> {  // fp16
+    static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                      0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        const f32x2 f = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
+    }
+    static __device__ __forceinline__ u32x2 tr_read(const uint8_t *lds_ptr) {
+        // the transposing read only moves 16-bit lanes around, so the bf16 flavour serves fp16 too
+        return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((SA_LDS bf16x4 *)lds_ptr));
+    }
+    static __device__ __forceinline__ u32x4 ones4() {
+        return u32x4{0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};
+    }
+};
+
+// Exchange a value between lane and lane^32 and combine: returns op(x[lane], x[lane^32]) in all lanes.
+__device__ __forceinline__ float half_swap_max(float x) {
+    const uint32_t u = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+constexpr float kNegInf = -__builtin_inff();
+
+// 16 bytes per lane from global memory (wave-uniform base + per-lane byte offset) straight into LDS:
+// lane i of the wave writes LDS address lds_addr + 16*i.
+// Issued through inline assembly on purpose: the compiler then does not track it, so it does not hold
+// back later LDS reads of the OTHER buffer until the transfer lands.  Whoever reads the destination
+// must execute "s_waitcnt vmcnt(0)" and a workgroup barrier first (the main loop does).
+__device__ __forceinline__ void dma16(const void *base, uint32_t lane_offset, uint32_t lds_addr) {
+    // the base is wave-uniform by construction; say so in a way the register allocator cannot miss
+    const uint64_t b = (uint64_t)(uintptr_t)base;
+    // (readfirstlane returns a signed int: widen through uint32_t, or the low half sign-extends)
+    const uint64_t ub = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b) |
+                        ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32)) << 32);
+    lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
+    asm volatile(
+        "s_mov_b32 m0, %2\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %0, %1"
+        :
+        : "v"(lane_offset), "s"(ub), "s"(lds_addr)
+        : "memory");  // m0 is written; nothing else in these kernels keeps a value in it
+}
+
+// Swizzles of the 16-byte pieces inside an LDS row.  Rows are stored unpadded (D*2 bytes) because a
+// direct global->LDS load writes 64 lanes x 16 bytes contiguously; instead the piece index is XORed
+// with a function of the row so that
+//   K: the 16 rows read together by one quarter-wave ds_read_b128 fall into 16 different bank groups,
+//   V: the 4 rows touched by one half-wave transposing read fall into 4 different 64-byte bank groups.
+template <int D>
+__device__ __forceinline__ int k_swizzle(int row) {
+    return D == 128 ? (row & 15) : ((row >> 1) & 7);
+}
+template <int D>
+__device__ __forceinline__ int v_swizzle(int row) {
+    return D == 128 ? 4 * (row & 3) : 4 * ((row >> 1) & 1);
+}
+
+// log2-domain slack before the running maximum is raised (and the accumulator rescaled).  Scores are
+// exponentiated against a reference value that may lag the true row maximum by up to this much, so
+// P stays <= 2^kMaxSlack; the final division by the row sum cancels the reference exactly.
+constexpr float kMaxSlack = 8.0f;
+
+// List entries kept in LDS per Q tile (8 KiB); longer lists are read from global memory per chunk.
+constexpr int kListCap = 2048;
+
+}  // namespace
+}  // namespace sa
