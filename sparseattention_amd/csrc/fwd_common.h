@@ -33,9 +33,18 @@ struct Elem<0> {  // bf16
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
                                                        0, 0, 0);
     }
+    // 16x16x32 product; lane l supplies row/column l%16 and the 8 contraction indices 8*(l/16)..+7, and
+    // receives column l%16, rows 4*(l/16)..+3
+    static __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                       0, 0, 0);
+    }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         const f32x2 f = {lo, hi};
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+    }
+    static __device__ __forceinline__ uint32_t scale2(uint32_t w, float s) {  // both halves times s, rounded again
+        return pack2(__uint_as_float(w << 16) * s, __uint_as_float(w & 0xffff0000u) * s);
     }
     static __device__ __forceinline__ u32x2 tr_read(const uint8_t *lds_ptr) {
         return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16((SA_LDS bf16x4 *)lds_ptr));
@@ -51,9 +60,17 @@ struct Elem<1> {  // fp16
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
                                                       0, 0);
     }
+    static __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                      0, 0);
+    }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         const f32x2 f = {lo, hi};
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
+    }
+    static __device__ __forceinline__ uint32_t scale2(uint32_t w, float s) {
+        const f16x2 h = __builtin_bit_cast(f16x2, w);
+        return pack2((float)h.x * s, (float)h.y * s);
     }
     static __device__ __forceinline__ u32x2 tr_read(const uint8_t *lds_ptr) {
         // the transposing read only moves 16-bit lanes around, so the bf16 flavour serves fp16 too

@@ -30,8 +30,33 @@ namespace sa {
 
 namespace {
 
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {  // f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
+
+// "At most n vector-memory operations of this wave still in flight", n a small run-time value.
+__device__ __forceinline__ void wait_vm_at_most(int n, int step) {
+    if (n <= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else if (n == 1) {
+        if (step == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+        else if (step == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        else if (step == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else {
+        if (step == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        else if (step == 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        else if (step == 8) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+}
+
 // MODE 0: BK = 16, MODE 1: BK = 32, MODE 2: BK >= 64 (runtime log2 in p.lbk).
-template <int DT, int D, int NW, int MODE>
+// NS: LDS stages per operand (2 or 4); chunks are fetched NS-1 ahead of the one being computed.
+template <int DT, int D, int NW, int MODE, int NS>
 __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(const FwdParams p) {
     using E = Elem<DT>;
     constexpr int ROWB = D * 2;                   // bytes per K/V row in LDS
@@ -44,8 +69,10 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
     static_assert(64 % (RPI * NW) == 0, "staging layout");
 
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-    // [K buf 0][K buf 1][V buf 0][V buf 1][first key column of every list entry, kListCap ints]
-    int *const ent = reinterpret_cast<int *>(smem + 2 * KBUF + 2 * VBUF);
+    static_assert(NS == 2 || NS == 4, "stage count");
+    constexpr int PD = NS - 1;  // fetch distance in chunks
+    // [K stage 0..NS-1][V stage 0..NS-1][first key column of every list entry, kListCap ints]
+    int *const ent = reinterpret_cast<int *>(smem + NS * KBUF + NS * VBUF);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, hh = lane >> 5;
@@ -79,12 +106,31 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         const uint16_t *qp = p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2] + 8 * hh;
 #pragma unroll
         for (int c = 0; c < D / 16; c++) qf[c] = *(const u32x4 *)(qp + 16 * c);
+        // The scale (softmax scale / ln 2) goes into Q once, so that the S MFMAs deliver exp2 arguments.
+#pragma unroll
+        for (int c = 0; c < D / 16; c++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) qf[c][e] = E::scale2(qf[c][e], p.scale);
     }
 
-    float m_run = kNegInf;  // reference value of the row's exponentials, in exp2 units (score * scale)
-    f32x16 acc_l;           // every element: running row sum of P for this lane's query (see the P.V loop)
+    // Online-softmax state of this lane's query row.  Exponentials are taken against a reference value m_ref
+    // (exp2 units).  The S MFMAs start from the accumulator -m_ref (neg_m: the same value in all 16 registers,
+    // one query per lane), so a score leaves the matrix unit as the exp2 argument itself.  raise_above is the
+    // largest such argument tolerated before m_ref moves: kMaxSlack, or "anything finite" until the row has
+    // seen its first attended key.
+    float m_ref = 0.f;
+    float raise_above = -3.0e38f;
+    f32x16 neg_m;
 #pragma unroll
-    for (int i = 0; i < 16; i++) acc_l[i] = 0.f;
+    for (int i = 0; i < 16; i++) neg_m[i] = 0.f;
+    // Running row sums of P, kept by a 16x16x32 MFMA whose B operand is P itself.  In that instruction lane l
+    // supplies column l%16 and key group l/16, so the P registers of query rows r and r+16 land in the same
+    // column; the A operand separates them again: its row i is all ones over the key groups of parity i&1 and
+    // zero elsewhere.  Result register 0 of lane l is then the row sum of query l%16 and register 1 that of
+    // query l%16 + 16; a lane reads the one that belongs to its own row.
+    f32x4 acc_l = {0.f, 0.f, 0.f, 0.f};
+    const uint32_t sel1 = (((lane >> 4) ^ lane) & 1) == 0 ? E::ones4().x : 0u;
+    const u32x4 sum_sel = {sel1, sel1, sel1, sel1};
     f32x16 acc[D / 32];
 #pragma unroll
     for (int db = 0; db < D / 32; db++)
@@ -171,33 +217,44 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         }
     };
 
-    // Global -> LDS for one chunk, without passing through registers.
-    auto stage_chunk = [&](int buf, const int(&col)[EPC]) {
+    // Global -> LDS for one chunk, without passing through registers: 2*NLD direct loads per wave (piece 2i is
+    // load i of K, piece 2i+1 load i of V).  A wave that issues them back to back sits at the issue stage until
+    // the address unit has taken them all, while every other wave of the CU does the same; the main loop
+    // therefore hands them out one at a time between the MFMA bundles of the chunk being computed.
+    struct StagePlan {
         const uint16_t *kp[EPC], *vp[EPC];  // first row of every list entry of the chunk (scalar registers)
+    };
+    auto plan_chunk = [&](const int(&col)[EPC], StagePlan &pl) {
 #pragma unroll
         for (int j = 0; j < EPC; j++) {
-            kp[j] = kbase + (int64_t)col[j] * p.ks[2];
-            vp[j] = vbase + (int64_t)col[j] * p.vs[2];
+            pl.kp[j] = kbase + (int64_t)col[j] * p.ks[2];
+            pl.vp[j] = vbase + (int64_t)col[j] * p.vs[2];
         }
+    };
+    auto stage_piece = [&](int buf, int piece, const StagePlan &pl) {
+        const int i = piece >> 1;
+        // rows [rbase, rbase + RPI) lie inside one list entry; when the rows of all waves of load i do, the
+        // entry is known at compile time
+        constexpr bool kEntryByLoad = MODE == 2 || RPI * NW <= (1 << LBKC);
+        const int rbase = RPI * (NW * i + wave_u);
+        const uint16_t *ks_ = pl.kp[0], *vs_ = pl.vp[0];
+        if constexpr (MODE != 2) {
+            const int j = kEntryByLoad ? ((RPI * NW * i) >> LBKC) : (rbase >> LBKC);
 #pragma unroll
-        for (int i = 0; i < NLD; i++) {
-            // rows [rbase, rbase + RPI) lie inside one list entry; when the rows of all waves of load i do,
-            // the entry is known at compile time
-            constexpr bool kEntryByLoad = MODE == 2 || RPI * NW <= (1 << LBKC);
-            const int rbase = RPI * (NW * i + wave_u);
-            const uint16_t *ks_ = kp[0], *vs_ = vp[0];
-            if constexpr (MODE != 2) {
-                const int j = kEntryByLoad ? ((RPI * NW * i) >> LBKC) : (rbase >> LBKC);
-#pragma unroll
-                for (int jj = 1; jj < EPC; jj++)
-                    if (j == jj) {
-                        ks_ = kp[jj];
-                        vs_ = vp[jj];
-                    }
-            }
-            dma16(ks_, ld_koff[i], lds0 + buf * KBUF + rbase * ROWB);
-            dma16(vs_, ld_voff[i], lds0 + 2 * KBUF + buf * VBUF + rbase * ROWB);
+            for (int jj = 1; jj < EPC; jj++)
+                if (j == jj) {
+                    ks_ = pl.kp[jj];
+                    vs_ = pl.vp[jj];
+                }
         }
+        if ((piece & 1) == 0) dma16(ks_, ld_koff[i], lds0 + buf * KBUF + rbase * ROWB);
+        else dma16(vs_, ld_voff[i], lds0 + NS * KBUF + buf * VBUF + rbase * ROWB);
+    };
+    auto stage_chunk = [&](int buf, const int(&col)[EPC]) {  // all pieces at once (prologue)
+        StagePlan pl;
+        plan_chunk(col, pl);
+#pragma unroll
+        for (int i = 0; i < 2 * NLD; i++) stage_piece(buf, i, pl);
     };
 
     // Mask bytes of this lane's eight 4-key groups in a chunk (non-zero byte = attended key).  Called for
@@ -240,20 +297,20 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         }
     };
 
-    auto compute = [&](auto buf_c, bool special, unsigned valid, const uint32_t(&mk)[2][4]) {
+    // One chunk from stage BUF.  When `fetch`, the pieces of the chunk planned in `pl` are sent to stage FBUF
+    // between the MFMA bundles of the S phase.
+    auto compute = [&](auto buf_c, bool special, unsigned valid, const uint32_t(&mk)[2][4], auto fbuf_c, bool fetch,
+                       const StagePlan &pl) {
         constexpr int BUF = decltype(buf_c)::value;
+        constexpr int FBUF = decltype(fbuf_c)::value;
         const uint8_t *kb_ = smem + BUF * KBUF;
-        const uint8_t *vb_ = smem + 2 * KBUF + BUF * VBUF;
+        const uint8_t *vb_ = smem + NS * KBUF + BUF * VBUF;
 
         // S^T = K . Q^T in bundles of two MFMAs (the two key blocks of d step c), operand reads kPfS bundles
         // ahead.  Within a bundle the MFMA that uses the younger read goes first, so one wait covers both.
         constexpr int NC = D / 16;
         constexpr int kPfS = 3;
         f32x16 s[2];
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) s[kb][i] = 0.f;
         u32x4 kf0[NC], kf1[NC];
         auto k_read = [&](int c) {
             kf0[c] = *(const u32x4 *)(kb_ + koff[c]);
@@ -264,9 +321,13 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int c = 0; c < NC; c++) {
-            s[1] = E::mfma(kf1[c], qf[c], s[1]);
-            s[0] = E::mfma(kf0[c], qf[c], s[0]);
+            s[1] = E::mfma(kf1[c], qf[c], c == 0 ? neg_m : s[1]);
+            s[0] = E::mfma(kf0[c], qf[c], c == 0 ? neg_m : s[0]);
             if (c + kPfS < NC) k_read(c + kPfS);
+            if (fetch) {
+#pragma unroll
+                for (int i = 2 * NLD * c / NC; i < 2 * NLD * (c + 1) / NC; i++) stage_piece(FBUF, i, pl);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
 
@@ -283,36 +344,45 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
                 }
         }
 
-        // Online softmax in exp2 units (sparse_attn_kernel.py:47-58), with a lagging reference value.
+        // Online softmax in exp2 units (sparse_attn_kernel.py:47-58), with a lagging reference value: s holds
+        // score*scale - m_ref.  Only when some row's largest argument exceeds raise_above does m_ref move.
         float mx = kNegInf;
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
             for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[kb][i]);
-        mx = half_swap_max(mx) * p.scale;
-        const bool raise = mx > m_run + kMaxSlack;  // also true for the first finite maximum (m_run = -inf)
+        mx = half_swap_max(mx);
+        const bool raise = mx > raise_above;  // false for rows without an attended key so far (mx = -inf)
         if (__builtin_amdgcn_ballot_w64(raise) != 0ull) {
-            const float m_new = raise ? mx : m_run;
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // m_new is finite wherever raise holds
-            const float a = raise ? alpha : 1.f;
-            m_run = m_new;
+            // rows that raise: m_ref += mx, the arguments drop by mx, what was accumulated shrinks by 2^-mx
+            // (nothing was accumulated if this is the row's first attended key: factor 0, not 2^-mx, which
+            // may be infinite)
+            const float delta = raise ? mx : 0.f;
+            const float a = raise ? (raise_above == kMaxSlack ? __builtin_amdgcn_exp2f(-mx) : 0.f) : 1.f;
+            m_ref += delta;
+            raise_above = raise ? kMaxSlack : raise_above;
 #pragma unroll
-            for (int i = 0; i < 16; i++) acc_l[i] *= a;
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) s[kb][i] -= delta;
+#pragma unroll
+            for (int i = 0; i < 16; i++) neg_m[i] = -m_ref;
+#pragma unroll
+            for (int i = 0; i < 2; i++) acc_l[i] *= a;  // the lane only ever reads the one of its own row
 #pragma unroll
             for (int db = 0; db < D / 32; db++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) acc[db][i] *= a;
         }
-        const float m_ref = m_run == kNegInf ? 0.f : m_run;  // keeps exp2(-inf - -inf) out of the picture
 
-        // P = exp2(S*scale - m_ref), rounded to the input dtype, and O^T += V^T . P^T.
+        // P = exp2(s), rounded to the input dtype, and O^T += V^T . P^T.
         // MFMA (key step kc, d block db) needs only the kc-th group of 8 P values, so the loop is a software
         // pipeline of bundles pinned by scheduling barriers: two MFMAs (d blocks 2h, 2h+1 of one key step) |
         // the transposing reads for a later bundle | half of the next key step's exponentials.
-        // The row sum comes from one more MFMA per key step whose A operand is all ones: every row of its
-        // result is sum_k P[k][q] over the 16 keys of the step, both lane halves included.  It therefore adds
-        // up the ROUNDED values, the ones that enter P.V, and the output is an exact convex combination of
-        // value rows (the reference sums the unrounded ones; the difference is bounded by the rounding of P).
+        // The row sum comes from one small MFMA per key step (see acc_l): it adds up the 16 keys of the step,
+        // both lane halves included, and it adds up the ROUNDED values, the ones that enter P.V, so the output
+        // is an exact convex combination of value rows (the reference sums the unrounded ones; the difference
+        // is bounded by the rounding of P).
         constexpr int NDB = D / 32;
         constexpr int NB = 4 * NDB / 2;  // bundles; bundle b: key step b / (NDB/2), d blocks 2*(b % (NDB/2)) + {0,1}
         constexpr int BPK = NDB / 2;     // bundles per key step
@@ -322,8 +392,8 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         auto p_values = [&](int kc, int first, int count) {
 #pragma unroll
             for (int i = first; i < first + count; i += 2) {
-                const float x0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kc >> 1][8 * (kc & 1) + i], p.scale, -m_ref));
-                const float x1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kc >> 1][8 * (kc & 1) + i + 1], p.scale, -m_ref));
+                const float x0 = __builtin_amdgcn_exp2f(s[kc >> 1][8 * (kc & 1) + i]);
+                const float x1 = __builtin_amdgcn_exp2f(s[kc >> 1][8 * (kc & 1) + i + 1]);
                 pw[4 * kc + (i >> 1)] = E::pack2(x0, x1);
             }
         };
@@ -350,7 +420,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
                 const int db = 2 * (b % BPK) + u, i = 2 * b + u;
                 acc[db] = E::mfma(u32x4{vlo[i].x, vlo[i].y, vhi[i].x, vhi[i].y}, pk4, acc[db]);
             }
-            if (b % BPK == BPK - 1) acc_l = E::mfma(E::ones4(), pk4, acc_l);
+            if (b % BPK == BPK - 1) acc_l = E::mfma16(sum_sel, pk4, acc_l);
             if (b + kPfV < NB) v_read(b + kPfV);
             if (kc + 1 < 4) p_values(kc + 1, PER * (b % BPK), PER);
             __builtin_amdgcn_sched_barrier(0);
@@ -369,52 +439,69 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
 
     if (T > 0) {
         int col[EPC];
-        unsigned valid, part, valid_a, valid_b = 0u;
-        uint32_t mk_a[2][4] = {}, mk_b[2][4] = {};
-        bool sp_a, sp_b = false;
+        unsigned valid, part;
+        uint32_t mk[2][2][4] = {};  // mask words of the chunk being computed / of the next one, by chunk parity
+        bool sp[2] = {false, false};
+        unsigned vl[2] = {0u, 0u};
         constexpr unsigned ALL = (1u << EPC) - 1u;
+        constexpr int kOpsPerChunk = 2 * NLD;  // direct loads per wave and chunk
         __syncthreads();  // the list in LDS is complete
-        chunk_entries(0, col, valid, part);
-        stage_chunk(0, col);
-        sp_a = part != 0u || valid != ALL;
-        valid_a = valid;
-        if (sp_a) load_mask(col, mk_a);
+        // prologue: chunks 0 .. PD-1 on their way, mask words of chunk 0
+        static_for<PD>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            if (j < T) {
+                chunk_entries(j, col, valid, part);
+                stage_chunk(j, col);
+                if constexpr (j == 0) {
+                    sp[0] = part != 0u || valid != ALL;
+                    vl[0] = valid;
+                    if (sp[0]) load_mask(col, mk[0]);
+                }
+            }
+        });
 #pragma unroll
         for (int c = 0; c < D / 16; c++) asm volatile("" ::"v"(qf[c]));
-        settle(mk_a);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        settle(mk[0]);
+        wait_vm_at_most((T < PD ? T : PD) - 1, kOpsPerChunk);  // chunk 0 has landed; later ones may be in flight
         __syncthreads();
-        // Two chunks per trip so that the LDS buffer index is a compile-time constant.
-        for (int t = 0; t < T; t += 2) {
-            if (t + 1 < T) {
-                chunk_entries(t + 1, col, valid, part);
-                stage_chunk(1, col);
-                sp_b = part != 0u || valid != ALL;
-                valid_b = valid;
-                if (sp_b) load_mask(col, mk_b);
-            }
-            compute(std::integral_constant<int, 0>{}, sp_a, valid_a, mk_a);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            settle(mk_b);
-            __syncthreads();
-            if (t + 1 < T) {
-                if (t + 2 < T) {
-                    chunk_entries(t + 2, col, valid, part);
-                    stage_chunk(0, col);
-                    sp_a = part != 0u || valid != ALL;
-                    valid_a = valid;
-                    if (sp_a) load_mask(col, mk_a);
+        // NS chunks per trip so that the LDS stage is a compile-time constant.  In front of chunk tc: every
+        // wave has finished chunk tc-1 (barrier), so its stage takes chunk tc+PD.
+        for (int t = 0; t < T; t += NS) {
+            static_for<NS>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                constexpr int cur = j & 1, nxt = cur ^ 1;
+                const int tc = t + j;
+                if (tc < T) {
+                    StagePlan pl;
+                    const bool fetch = tc + PD < T;
+                    if constexpr (PD > 1) {
+                        chunk_entries(fetch ? tc + PD : tc, col, valid, part);
+                        plan_chunk(col, pl);
+                    }
+                    sp[nxt] = false;
+                    if (tc + 1 < T) {
+                        chunk_entries(tc + 1, col, valid, part);
+                        if constexpr (PD == 1) plan_chunk(col, pl);
+                        sp[nxt] = part != 0u || valid != ALL;
+                        vl[nxt] = valid;
+                        if (sp[nxt]) load_mask(col, mk[nxt]);
+                    } else if constexpr (PD == 1) {
+                        plan_chunk(col, pl);  // not used (fetch is false); keeps the plan defined
+                    }
+                    compute(jc, sp[cur], vl[cur], mk[cur], std::integral_constant<int, (j + PD) % NS>{}, fetch, pl);
+                    // chunk tc+1 must have landed (and its mask words, the youngest loads, when it has any);
+                    // chunks tc+2 .. tc+PD may stay in flight
+                    const int last = tc + PD < T ? tc + PD : T - 1;
+                    wait_vm_at_most(sp[nxt] ? 0 : last - (tc + 1), kOpsPerChunk);
+                    settle(mk[nxt]);
+                    __syncthreads();
                 }
-                compute(std::integral_constant<int, 1>{}, sp_b, valid_b, mk_b);
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                settle(mk_a);
-                __syncthreads();
-            }
+            });
         }
     }
 
     // Epilogue: O = acc / l (sparse_attn_kernel.py:144); rows that attended to nothing give 0.
-    const float l_tot = acc_l[0];
+    const float l_tot = l32 < 16 ? acc_l[0] : acc_l[1];
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     uint16_t *orow = p.o + b * p.os[0] + h * p.os[1] + (int64_t)qrow * p.os[2] + 4 * hh;
 #pragma unroll
@@ -429,8 +516,10 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
 
 template <int DT, int D, int NW, int MODE>
 hipError_t launch_one(const FwdParams &p, hipStream_t stream) {
-    constexpr int smem = 4 * 64 * D * 2 + kListCap * 4;  // two K and two V buffers of 64 rows + the list
-    auto kern = sparse_fwd_kernel<DT, D, NW, MODE>;
+    // Eight waves fill a CU's register file on their own, so that workgroup can have most of the LDS: 4 stages.
+    constexpr int NS = NW == 8 ? 4 : 2;
+    constexpr int smem = 2 * NS * 64 * D * 2 + kListCap * 4;  // NS stages of 64 rows for K and for V + the list
+    auto kern = sparse_fwd_kernel<DT, D, NW, MODE, NS>;
     static bool attr_set = false;  // benign race: every thread sets the same value
     if (!attr_set) {
         const hipError_t e =
