@@ -56,7 +56,9 @@ __device__ __forceinline__ void wait_vm_at_most(int n, int step) {
 
 // MODE 0: BK = 16, MODE 1: BK = 32, MODE 2: BK >= 64 (runtime log2 in p.lbk).
 // NS: LDS stages per operand (2 or 4); chunks are fetched NS-1 ahead of the one being computed.
-template <int DT, int D, int NW, int MODE, int NS>
+// PP: the two waves that share a SIMD (w and w+4 of an 8-wave workgroup) run half a chunk apart, one in its
+// S phase while the other is in its P.V phase (see the main loop).
+template <int DT, int D, int NW, int MODE, int NS, bool PP>
 __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(const FwdParams p) {
     using E = Elem<DT>;
     constexpr int ROWB = D * 2;                   // bytes per K/V row in LDS
@@ -79,13 +81,16 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
 
     // Workgroup -> (b, h, Q tile).  Hardware hands consecutive workgroup ids to the 8 XCDs in turn; the
     // remap gives each XCD a contiguous range of the (b,h)-major order so that the Q tiles sharing one
-    // K/V plane run on the XCD whose L2 already holds it.  Within a plane the last Q tile goes first
-    // (under causal-like masks it has the longest list).
+    // K/V plane run on the XCD whose L2 already holds it.  Planes are taken two at a time with their Q tiles
+    // interleaved, last Q tile first (under causal-like masks it has the longest list): the slots that finish
+    // the short tiles of one pair then pick up the long tiles of the next, which evens out the load.
     const int total = gridDim.x, per = total >> 3;
     int lin = blockIdx.x;
     if (lin < (per << 3)) lin = (lin & 7) * per + (lin >> 3);
-    const int bh = lin / p.nQ;
-    const int qt = p.nQ - 1 - (lin - bh * p.nQ);
+    const int pair = lin / (2 * p.nQ), r = lin - pair * 2 * p.nQ;
+    const bool paired = 2 * pair + 1 < p.B * p.H;  // the last plane of an odd count goes alone
+    const int bh = 2 * pair + (paired ? (r & 1) : 0);
+    const int qt = p.nQ - 1 - (paired ? (r >> 1) : r);
     const int b = bh / p.H, h = bh - b * p.H;
 
     const uint16_t *kbase = p.k + b * p.ks[0] + h * p.ks[1];
@@ -297,20 +302,18 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         }
     };
 
-    // One chunk from stage BUF.  When `fetch`, the pieces of the chunk planned in `pl` are sent to stage FBUF
-    // between the MFMA bundles of the S phase.
-    auto compute = [&](auto buf_c, bool special, unsigned valid, const uint32_t(&mk)[2][4], auto fbuf_c, bool fetch,
-                       const StagePlan &pl) {
+    // One chunk from stage BUF, in two phases.
+    // S phase: s = K . Q^T - m_ref.  When `fetch`, the pieces of the chunk planned in `pl` are sent to stage
+    // FBUF between its MFMA bundles.
+    auto phase_s = [&](auto buf_c, f32x16(&s)[2], auto fbuf_c, bool fetch, const StagePlan &pl) {
         constexpr int BUF = decltype(buf_c)::value;
         constexpr int FBUF = decltype(fbuf_c)::value;
         const uint8_t *kb_ = smem + BUF * KBUF;
-        const uint8_t *vb_ = smem + NS * KBUF + BUF * VBUF;
 
         // S^T = K . Q^T in bundles of two MFMAs (the two key blocks of d step c), operand reads kPfS bundles
         // ahead.  Within a bundle the MFMA that uses the younger read goes first, so one wait covers both.
         constexpr int NC = D / 16;
         constexpr int kPfS = 3;
-        f32x16 s[2];
         u32x4 kf0[NC], kf1[NC];
         auto k_read = [&](int c) {
             kf0[c] = *(const u32x4 *)(kb_ + koff[c]);
@@ -330,7 +333,11 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-
+    };
+    // P.V phase: mask, online softmax, O^T += V^T . P^T.
+    auto phase_pv = [&](auto buf_c, f32x16(&s)[2], bool special, unsigned valid, const uint32_t(&mk)[2][4]) {
+        constexpr int BUF = decltype(buf_c)::value;
+        const uint8_t *vb_ = smem + NS * KBUF + BUF * VBUF;
         if (special) {
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
@@ -437,7 +444,73 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
             for (int g = 0; g < 4; g++) asm volatile("" ::"v"(mk[kb][g]));
     };
 
-    if (T > 0) {
+    if constexpr (PP) {
+        // Ping-pong schedule.  Every wave runs  barrier | S phase | barrier | P.V phase  per chunk; waves 4..7
+        // enter the sequence one barrier later than waves 0..3, so between two barriers one wave of each SIMD
+        // issues the MFMA-only S phase while the other does softmax and P.V, and the matrix unit always has a
+        // taker.  Chunk t is needed first by waves 0..3 after barrier 2t and last by waves 4..7 before barrier
+        // 2t+3; it is fetched two chunks ahead into a ring of 4 stages, whose slot was given up before barrier
+        // 2t-1.  Before arriving at barrier 2t every wave has waited for its own pieces of chunk t.
+        static_assert(!PP || (NW == 8 && NS == 4), "ping-pong layout");
+        if (T > 0) {
+            const int late = wave_u >> 2;  // 1: this wave runs half a chunk behind
+            int col[EPC], coln[EPC];       // entries of the chunk at hand / of the next chunk to look at
+            unsigned valid, part, validn = 0u, partn = 0u;
+            uint32_t mk[2][2][4] = {};
+            bool sp[2] = {false, false};
+            unsigned vl[2] = {0u, 0u};
+            constexpr unsigned ALL = (1u << EPC) - 1u;
+            constexpr int kOpsPerChunk = 2 * NLD;
+            __syncthreads();  // the list in LDS is complete
+            chunk_entries(0, col, valid, part);
+            stage_chunk(0, col);
+            sp[0] = part != 0u || valid != ALL;
+            vl[0] = valid;
+            if (sp[0]) load_mask(col, mk[0]);
+#pragma unroll
+            for (int j = 0; j < EPC; j++) coln[j] = col[j];
+            if (1 < T) {
+                chunk_entries(1, coln, validn, partn);
+                stage_chunk(1, coln);
+            }
+#pragma unroll
+            for (int c = 0; c < D / 16; c++) asm volatile("" ::"v"(qf[c]));
+            if (sp[0]) settle(mk[0]);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (late) __syncthreads();
+            for (int t = 0; t < T; t += NS) {
+                static_for<NS>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    constexpr int cur = j & 1, nxt = cur ^ 1;
+                    const int tc = t + j;
+                    if (tc < T) {
+                        // own pieces of chunk tc have landed; chunk tc+1 may be in flight
+                        wait_vm_at_most((tc + 1 < T ? tc + 1 : T - 1) - tc, kOpsPerChunk);
+                        if (sp[cur]) settle(mk[cur]);
+                        __syncthreads();
+                        sp[nxt] = false;
+                        if (tc + 1 < T) {  // coln: entries of chunk tc+1
+                            sp[nxt] = partn != 0u || validn != ALL;
+                            vl[nxt] = validn;
+                            if (sp[nxt]) load_mask(coln, mk[nxt]);
+                        }
+                        const bool fetch = tc + 2 < T;
+                        if (fetch) chunk_entries(tc + 2, coln, validn, partn);
+                        StagePlan pl;
+                        plan_chunk(coln, pl);
+                        f32x16 s[2];
+                        phase_s(jc, s, std::integral_constant<int, (j + 2) % NS>{}, fetch, pl);
+                        // own pieces of chunk tc+1 have landed; chunk tc+2 may be in flight
+                        wait_vm_at_most((tc + 2 < T ? tc + 2 : T - 1) - (tc + 1), kOpsPerChunk);
+                        __syncthreads();
+                        phase_pv(jc, s, sp[cur], vl[cur], mk[cur]);
+                    }
+                });
+            }
+            if (!late) __syncthreads();
+        }
+    } else if (T > 0) {
         int col[EPC];
         unsigned valid, part;
         uint32_t mk[2][2][4] = {};  // mask words of the chunk being computed / of the next one, by chunk parity
@@ -461,7 +534,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         });
 #pragma unroll
         for (int c = 0; c < D / 16; c++) asm volatile("" ::"v"(qf[c]));
-        settle(mk[0]);
+        if (sp[0]) settle(mk[0]);
         wait_vm_at_most((T < PD ? T : PD) - 1, kOpsPerChunk);  // chunk 0 has landed; later ones may be in flight
         __syncthreads();
         // NS chunks per trip so that the LDS stage is a compile-time constant.  In front of chunk tc: every
@@ -488,12 +561,14 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
                     } else if constexpr (PD == 1) {
                         plan_chunk(col, pl);  // not used (fetch is false); keeps the plan defined
                     }
-                    compute(jc, sp[cur], vl[cur], mk[cur], std::integral_constant<int, (j + PD) % NS>{}, fetch, pl);
+                    f32x16 s[2];
+                    phase_s(jc, s, std::integral_constant<int, (j + PD) % NS>{}, fetch, pl);
+                    phase_pv(jc, s, sp[cur], vl[cur], mk[cur]);
                     // chunk tc+1 must have landed (and its mask words, the youngest loads, when it has any);
                     // chunks tc+2 .. tc+PD may stay in flight
                     const int last = tc + PD < T ? tc + PD : T - 1;
                     wait_vm_at_most(sp[nxt] ? 0 : last - (tc + 1), kOpsPerChunk);
-                    settle(mk[nxt]);
+                    if (sp[nxt]) settle(mk[nxt]);
                     __syncthreads();
                 }
             });
@@ -519,7 +594,7 @@ hipError_t launch_one(const FwdParams &p, hipStream_t stream) {
     // Eight waves fill a CU's register file on their own, so that workgroup can have most of the LDS: 4 stages.
     constexpr int NS = NW == 8 ? 4 : 2;
     constexpr int smem = 2 * NS * 64 * D * 2 + kListCap * 4;  // NS stages of 64 rows for K and for V + the list
-    auto kern = sparse_fwd_kernel<DT, D, NW, MODE, NS>;
+    auto kern = sparse_fwd_kernel<DT, D, NW, MODE, NS, NW == 8>;
     static bool attr_set = false;  // benign race: every thread sets the same value
     if (!attr_set) {
         const hipError_t e =
