@@ -187,39 +187,51 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
             ent[e] = MODE == 2 ? (idx << p.lbk) : (idx << LBKC);
         }
     }
-    auto entry_col = [&](int e) -> int {  // wave-uniform result, kept in a scalar register
-        int c;
-        if (list_in_lds) {
-            c = ent[e];
-        } else {
-            const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
-            c = MODE == 2 ? (idx << p.lbk) : (idx << LBKC);
-        }
-        return __builtin_amdgcn_readfirstlane(c);
+    // First key column of every list entry in chunk t (t < T), plus which entries exist / are partial, in two
+    // steps: entries_read issues the reads of the list (the values are the same in all lanes), entries_use turns
+    // them into scalars.  The main loop reads the entries of a chunk one iteration before it needs them, so
+    // that no wave waits for the list.
+    auto entry_read = [&](int e) -> int {
+        if (list_in_lds) return ent[e];
+        const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
+        return MODE == 2 ? (idx << p.lbk) : (idx << LBKC);
     };
-
-    // First key column of every list entry in chunk t (t < T), plus which entries exist / are partial.
-    auto chunk_entries = [&](int t, int(&col)[EPC], unsigned &valid, unsigned &part) {
+    auto entries_read = [&](int t, int(&raw)[EPC]) {
+        if constexpr (MODE == 2) {
+            raw[0] = entry_read(t >> (p.lbk - 6));
+        } else {
+#pragma unroll
+            for (int j = 0; j < EPC; j++) {
+                const int e = t * EPC + j;
+                raw[j] = entry_read(e < NE ? e : t * EPC);  // absent entries re-read the chunk's first one;
+            }                                                // their scores are discarded
+        }
+    };
+    auto entries_use = [&](int t, const int(&raw)[EPC], int(&col)[EPC], unsigned &valid, unsigned &part) {
         valid = 0u;
         part = 0u;
         if constexpr (MODE == 2) {
             const int sh = p.lbk - 6;
             const int e = t >> sh, sub = t & ((1 << sh) - 1);
-            col[0] = entry_col(e) + (sub << 6);
+            col[0] = __builtin_amdgcn_readfirstlane(raw[0]) + (sub << 6);
             valid = 1u;
             part = e >= F ? 1u : 0u;
         } else {
 #pragma unroll
             for (int j = 0; j < EPC; j++) {
                 const int e = t * EPC + j;
-                // absent entries re-read the chunk's first one; their scores are discarded
-                col[j] = entry_col(e < NE ? e : t * EPC);
+                col[j] = __builtin_amdgcn_readfirstlane(raw[j]);
                 if (e < NE) {
                     valid |= 1u << j;
                     if (e >= F) part |= 1u << j;
                 }
             }
         }
+    };
+    auto chunk_entries = [&](int t, int(&col)[EPC], unsigned &valid, unsigned &part) {
+        int raw[EPC];
+        entries_read(t, raw);
+        entries_use(t, raw, col, valid, part);
     };
 
     // Global -> LDS for one chunk, without passing through registers: 2*NLD direct loads per wave (piece 2i is
@@ -475,6 +487,8 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
             }
 #pragma unroll
             for (int c = 0; c < D / 16; c++) asm volatile("" ::"v"(qf[c]));
+            int raw[EPC] = {};  // list entries of the chunk after next, read ahead
+            if (2 < T) entries_read(2, raw);
             if (sp[0]) settle(mk[0]);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
@@ -496,7 +510,10 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
                             if (sp[nxt]) load_mask(coln, mk[nxt]);
                         }
                         const bool fetch = tc + 2 < T;
-                        if (fetch) chunk_entries(tc + 2, coln, validn, partn);
+                        if (fetch) {
+                            entries_use(tc + 2, raw, coln, validn, partn);
+                            if (tc + 3 < T) entries_read(tc + 3, raw);
+                        }
                         StagePlan pl;
                         plan_chunk(coln, pl);
                         f32x16 s[2];
@@ -534,6 +551,8 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         });
 #pragma unroll
         for (int c = 0; c < D / 16; c++) asm volatile("" ::"v"(qf[c]));
+        int raw[EPC] = {};  // list entries of the next chunk, read ahead
+        if (PD == 1 && 1 < T) entries_read(1, raw);
         if (sp[0]) settle(mk[0]);
         wait_vm_at_most((T < PD ? T : PD) - 1, kOpsPerChunk);  // chunk 0 has landed; later ones may be in flight
         __syncthreads();
@@ -553,7 +572,12 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
                     }
                     sp[nxt] = false;
                     if (tc + 1 < T) {
-                        chunk_entries(tc + 1, col, valid, part);
+                        if constexpr (PD == 1) {
+                            entries_use(tc + 1, raw, col, valid, part);
+                            if (tc + 2 < T) entries_read(tc + 2, raw);
+                        } else {
+                            chunk_entries(tc + 1, col, valid, part);
+                        }
                         if constexpr (PD == 1) plan_chunk(col, pl);
                         sp[nxt] = part != 0u || valid != ALL;
                         vl[nxt] = valid;
