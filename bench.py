@@ -32,7 +32,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E peak, GB/s
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this script and scaled by
 # the readings of a 1 GiB device copy in the same run (--calibrate-copy).  The summaries with the commands
 # are profiles/sparse_fwd_kernel_causal_B8H32S4096D128.txt and profiles/mask_classify_kernels_mask_32768x32768.txt.
-TRAFFIC_FWD_CAUSAL_BYTES = 1.2284e9      # 915.4 MiB read + 256.1 MiB written
+TRAFFIC_FWD_CAUSAL_BYTES = 1.3256e9      # 1007.6 MiB read + 256.6 MiB written
 TRAFFIC_CLASSIFY_1GIB_BYTES = 1.0745e9   # 1,048,648 + 331 KiB read, 256 + 45.5 KiB written
 
 B, H, S, D = 8, 32, 4096, 128
