@@ -9,7 +9,7 @@ Same Python surface as tomatillos/sparseattention for its one hot path:
 The device work is done by hand-written gfx950 HIP kernels in ``libsparseattn_hip.so``
 behind the C ABI of ``include/sparseattn.h``.
 """
-from .mask_utils import MaskMetadata, compute_mask_kernel, compute_mask_slow
+from .mask_utils import MaskMetadata, compute_mask_kernel, compute_mask_slow, select_block_sizes
 from .sparse_attn_kernel import sparse_attention
 
-__all__ = ["MaskMetadata", "compute_mask_kernel", "compute_mask_slow", "sparse_attention"]
+__all__ = ["MaskMetadata", "compute_mask_kernel", "compute_mask_slow", "select_block_sizes", "sparse_attention"]

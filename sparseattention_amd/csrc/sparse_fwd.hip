@@ -346,8 +346,10 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    // P.V phase: mask, online softmax, O^T += V^T . P^T.
-    auto phase_pv = [&](auto buf_c, f32x16(&s)[2], bool special, unsigned valid, const uint32_t(&mk)[2][4]) {
+    // P.V phase: mask, online softmax, O^T += V^T . P^T.  between(b, NB) is called once per MFMA bundle b of NB;
+    // the main loop uses it to spread scalar bookkeeping over the phase, where it hides behind the MFMAs.
+    auto phase_pv = [&](auto buf_c, f32x16(&s)[2], bool special, unsigned valid, const uint32_t(&mk)[2][4],
+                        auto &&between) {
         constexpr int BUF = decltype(buf_c)::value;
         const uint8_t *vb_ = smem + NS * KBUF + BUF * VBUF;
         if (special) {
@@ -442,6 +444,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
             if (b % BPK == BPK - 1) acc_l = E::mfma16(sum_sel, pk4, acc_l);
             if (b + kPfV < NB) v_read(b + kPfV);
             if (kc + 1 < 4) p_values(kc + 1, PER * (b % BPK), PER);
+            between(b, NB);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -521,78 +524,75 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
                         // own pieces of chunk tc+1 have landed; chunk tc+2 may be in flight
                         wait_vm_at_most((tc + 2 < T ? tc + 2 : T - 1) - (tc + 1), kOpsPerChunk);
                         __syncthreads();
-                        phase_pv(jc, s, sp[cur], vl[cur], mk[cur]);
+                        phase_pv(jc, s, sp[cur], vl[cur], mk[cur], [](int, int) {});
                     }
                 });
             }
             if (!late) __syncthreads();
         }
     } else if (T > 0) {
-        int col[EPC];
+        static_assert(PP || NS == 2, "two stages: the chunk being computed and the one being fetched");
+        int col[EPC], coln[EPC];  // entries of chunk 0 / of the chunk that the current iteration fetches
         unsigned valid, part;
         uint32_t mk[2][2][4] = {};  // mask words of the chunk being computed / of the next one, by chunk parity
         bool sp[2] = {false, false};
         unsigned vl[2] = {0u, 0u};
         constexpr unsigned ALL = (1u << EPC) - 1u;
-        constexpr int kOpsPerChunk = 2 * NLD;  // direct loads per wave and chunk
+        StagePlan pl;  // where the chunk fetched by the current iteration comes from
         __syncthreads();  // the list in LDS is complete
-        // prologue: chunks 0 .. PD-1 on their way, mask words of chunk 0
-        static_for<PD>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            if (j < T) {
-                chunk_entries(j, col, valid, part);
-                stage_chunk(j, col);
-                if constexpr (j == 0) {
-                    sp[0] = part != 0u || valid != ALL;
-                    vl[0] = valid;
-                    if (sp[0]) load_mask(col, mk[0]);
-                }
-            }
-        });
+        chunk_entries(0, col, valid, part);
+        stage_chunk(0, col);
+        sp[0] = part != 0u || valid != ALL;
+        vl[0] = valid;
+        if (sp[0]) load_mask(col, mk[0]);
+        chunk_entries(1 < T ? 1 : 0, coln, valid, part);
+        sp[1] = 1 < T && (part != 0u || valid != ALL);
+        vl[1] = valid;
+        plan_chunk(coln, pl);
+        int raw[EPC];  // list entries of the chunk after next, read ahead
+        entries_read(2 < T ? 2 : T - 1, raw);
 #pragma unroll
         for (int c = 0; c < D / 16; c++) asm volatile("" ::"v"(qf[c]));
-        int raw[EPC] = {};  // list entries of the next chunk, read ahead
-        if (PD == 1 && 1 < T) entries_read(1, raw);
         if (sp[0]) settle(mk[0]);
-        wait_vm_at_most((T < PD ? T : PD) - 1, kOpsPerChunk);  // chunk 0 has landed; later ones may be in flight
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        // NS chunks per trip so that the LDS stage is a compile-time constant.  In front of chunk tc: every
-        // wave has finished chunk tc-1 (barrier), so its stage takes chunk tc+PD.
-        for (int t = 0; t < T; t += NS) {
-            static_for<NS>([&](auto jc) {
+        // Two chunks per trip so that the LDS stage is a compile-time constant.  Iteration tc computes chunk tc
+        // while chunk tc+1 is fetched (its pieces go out between the S bundles) and, during the P.V phase, turns
+        // the list entries of chunk tc+2 into the fetch plan of the next iteration.  Indices past the last chunk
+        // are clamped to it: the values are computed and never used.
+        for (int t = 0; t < T; t += 2) {
+            static_for<2>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
                 constexpr int cur = j & 1, nxt = cur ^ 1;
                 const int tc = t + j;
                 if (tc < T) {
-                    StagePlan pl;
-                    const bool fetch = tc + PD < T;
-                    if constexpr (PD > 1) {
-                        chunk_entries(fetch ? tc + PD : tc, col, valid, part);
-                        plan_chunk(col, pl);
-                    }
-                    sp[nxt] = false;
-                    if (tc + 1 < T) {
-                        if constexpr (PD == 1) {
-                            entries_use(tc + 1, raw, col, valid, part);
-                            if (tc + 2 < T) entries_read(tc + 2, raw);
-                        } else {
-                            chunk_entries(tc + 1, col, valid, part);
-                        }
-                        if constexpr (PD == 1) plan_chunk(col, pl);
-                        sp[nxt] = part != 0u || valid != ALL;
-                        vl[nxt] = valid;
-                        if (sp[nxt]) load_mask(col, mk[nxt]);
-                    } else if constexpr (PD == 1) {
-                        plan_chunk(col, pl);  // not used (fetch is false); keeps the plan defined
-                    }
+                    const bool fetch = tc + 1 < T;
+                    if (sp[nxt]) load_mask(coln, mk[nxt]);
                     f32x16 s[2];
-                    phase_s(jc, s, std::integral_constant<int, (j + PD) % NS>{}, fetch, pl);
-                    phase_pv(jc, s, sp[cur], vl[cur], mk[cur]);
-                    // chunk tc+1 must have landed (and its mask words, the youngest loads, when it has any);
-                    // chunks tc+2 .. tc+PD may stay in flight
-                    const int last = tc + PD < T ? tc + PD : T - 1;
-                    wait_vm_at_most(sp[nxt] ? 0 : last - (tc + 1), kOpsPerChunk);
+                    phase_s(jc, s, std::integral_constant<int, nxt>{}, fetch, pl);
+                    const int t2 = tc + 2 < T ? tc + 2 : T - 1, t3 = tc + 3 < T ? tc + 3 : T - 1;
+                    int col2[EPC];
+                    unsigned valid2 = 0u, part2 = 0u;
+                    StagePlan pl2;
+                    phase_pv(jc, s, sp[cur], vl[cur], mk[cur], [&](int b, int nb) {
+                        const int per = (2 * EPC + nb - 1) / nb;  // plan entries per bundle
+                        if (b == 0) entries_use(t2, raw, col2, valid2, part2);
+#pragma unroll
+                        for (int i = b * per; i < (b + 1) * per && i < 2 * EPC; i++) {
+                            if (i & 1) pl2.vp[i >> 1] = vbase + (int64_t)col2[i >> 1] * p.vs[2];
+                            else pl2.kp[i >> 1] = kbase + (int64_t)col2[i >> 1] * p.ks[2];
+                        }
+                        if (b == nb - 1) entries_read(t3, raw);
+                    });
+                    pl = pl2;
+#pragma unroll
+                    for (int e = 0; e < EPC; e++) coln[e] = col2[e];
+                    // chunk tc+2 will be computed from the slot of chunk tc
+                    const bool sp2 = tc + 2 < T && (part2 != 0u || valid2 != ALL);
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // chunk tc+1 and its mask words have landed
                     if (sp[nxt]) settle(mk[nxt]);
+                    sp[cur] = sp2;
+                    vl[cur] = valid2;
                     __syncthreads();
                 }
             });

@@ -104,3 +104,45 @@ def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int) -> MaskM
         # only to work queued after them on the same stream, so dropping the reference here is safe
         del workspace
     return MaskMetadata(fid, fl, pid, pl)
+
+
+# Tile sizes tried by select_block_sizes, and what one executed mask entry costs at each BLOCK_Q relative to
+# BLOCK_Q = 128 (measured on MI355X with every tile executed, B8 H32 S4096 D128 bf16; BLOCK_K does not enter:
+# the forward consumes keys in chunks of 64 whatever the tile width).
+DEFAULT_TILE_CANDIDATES = ((128, 32), (128, 64), (128, 128), (64, 32), (64, 64), (256, 32), (256, 64))
+RELATIVE_COST_PER_ENTRY = {32: 1.55, 64: 1.2, 128: 1.0, 256: 1.05}
+
+
+def select_block_sizes(mask: torch.Tensor, candidates=DEFAULT_TILE_CANDIDATES, partial_cost: float = 1.25):
+    """Choose the tile sizes that leave the least attention work for this mask.
+
+    The reference lists this as future work ("changing blocksizes ... to maximise the number of totally
+    masked-out blocks", README.md:64).  Every candidate (BLOCK_Q, BLOCK_K) that divides the mask is
+    classified (on the GPU when the mask lives there, else with compute_mask_slow) and priced as
+
+        (full tiles + partial_cost * partial tiles) * BLOCK_Q * BLOCK_K * RELATIVE_COST_PER_ENTRY[BLOCK_Q]
+
+    summed over the distinct mask planes; partial tiles cost more because their mask is read and applied.
+    Returns ``(BLOCK_Q, BLOCK_K, metadata, report)``: the cheapest candidate, its MaskMetadata (ready to pass
+    to sparse_attention) and the list of ``(BLOCK_Q, BLOCK_K, full_tiles, partial_tiles, cost)`` rows.
+    Reads the counts back to the host, so it synchronises with the device: call it once per mask.
+    """
+    if mask.dim() != 4:
+        raise ValueError(f"mask must be [B,H,Sq,Sk] (got {tuple(mask.shape)})")
+    B, H, Sq, Sk = mask.shape
+    classify = compute_mask_kernel if mask.is_cuda else compute_mask_slow
+    best, report = None, []
+    for BQ, BK in candidates:
+        if Sq % BQ or Sk % BK:
+            continue
+        md = classify(mask, BQ, BK)
+        # broadcast planes hold the same counts: the sum over the expanded view weights every plane equally
+        full = int(md.unmasked_lens.sum())
+        part = int(md.masked_lens.sum())
+        cost = (full + partial_cost * part) * BQ * BK * RELATIVE_COST_PER_ENTRY.get(BQ, 1.0)
+        report.append((BQ, BK, full, part, cost))
+        if best is None or cost < best[0]:
+            best = (cost, BQ, BK, md)
+    if best is None:
+        raise ValueError(f"no candidate tile size divides a mask of shape {tuple(mask.shape)}")
+    return best[1], best[2], best[3], report
