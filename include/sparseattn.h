@@ -8,6 +8,10 @@
  *                             (sparseattention/mask_utils.py:85-107, kernel :47-82)
  *   sa_sparse_attention_fwd   replaces the launch in sparse_attention
  *                             (sparseattention/sparse_attn_kernel.py:149-185, kernels :10-63, :74-146)
+ *   sa_mask_pack_partial, sa_sparse_attention_fwd_packed
+ *                             an optional faster route for the PARTIAL tiles: their mask entries are
+ *                             packed to one bit each once per mask, and the forward reads those bits
+ *                             instead of the mask tile loads of sparse_attn_kernel.py:42-46
  *
  * Conventions
  *   - All pointers are DEVICE pointers owned by the caller.  The library allocates nothing,
@@ -32,7 +36,7 @@
 extern "C" {
 #endif
 
-#define SA_ABI_VERSION 1
+#define SA_ABI_VERSION 2
 
 enum sa_status {
     SA_OK = 0,
@@ -111,6 +115,50 @@ int sa_sparse_attention_fwd(const void *q, const int64_t q_strides[4], const voi
                             const int64_t part_ids_strides[4], const int32_t *part_lens,
                             const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int D, int BQ, int BK,
                             int dtype, float sm_scale_log2, void *stream);
+
+/*
+ * Bytes of the buffer sa_mask_pack_partial fills: Sq*Sk/8 for every DISTINCT mask plane (room for every
+ * tile being PARTIAL, so that no count has to be read back to the host).  Returns 0 on invalid arguments
+ * (BK must be a multiple of 8).
+ */
+size_t sa_mask_pack_partial_bytes(const int64_t mask_strides[4], int B, int H, int Sq, int Sk, int BQ, int BK);
+
+/*
+ * One bit per mask entry of every PARTIAL tile.  No counterpart in the reference, which re-reads the bool
+ * tile in every forward (sparse_attn_kernel.py:42-46); the reference README lists cheaper mask storage as
+ * an open problem (README.md:12, :63).
+ *
+ *   mask, part_ids, part_lens   as in sa_mask_classify, whose outputs the two lists must be (run on the
+ *                               same stream before this call).
+ *   packed           device buffer of sa_mask_pack_partial_bytes(...) bytes.  For the distinct plane
+ *                    (b, h) the tile that is entry `slot` of the PARTIAL list of Q tile `qt` lies at
+ *                        packed + b*packed_strides[0] + h*packed_strides[1] + (qt*(Sk/BK) + slot) * BQ*BK/8
+ *                    as BQ*BK/8 bytes, rows first: entry (r, c) of the tile is bit (c & 7) of byte
+ *                    (r*BK + c) >> 3, set when the mask byte is non-zero.  Slots >= the count are left
+ *                    untouched.
+ *   packed_strides   bytes between planes along b and h; give 0 where the mask stride is 0 (that
+ *                    dimension is then packed once).
+ */
+int sa_mask_pack_partial(const uint8_t *mask, const int64_t mask_strides[4], int B, int H, int Sq, int Sk, int BQ,
+                         int BK, const int32_t *part_ids, const int64_t part_ids_strides[4],
+                         const int32_t *part_lens, const int64_t part_lens_strides[3], uint8_t *packed,
+                         const int64_t packed_strides[2], void *stream);
+
+/*
+ * sa_sparse_attention_fwd with the PARTIAL tiles' mask entries taken from `packed` (the output of
+ * sa_mask_pack_partial for the same mask, tile sizes and lists; packed_strides may be 0 on broadcast
+ * dimensions).  `mask` is not read and may be NULL, so the bool tensor can be released once the lists and
+ * the packed bits exist.  Results are bit-identical to sa_sparse_attention_fwd.
+ */
+int sa_sparse_attention_fwd_packed(const void *q, const int64_t q_strides[4], const void *k,
+                                   const int64_t k_strides[4], const void *v, const int64_t v_strides[4], void *o,
+                                   const int64_t o_strides[4], const uint8_t *mask, const int64_t mask_strides[4],
+                                   const int32_t *full_ids, const int64_t full_ids_strides[4],
+                                   const int32_t *full_lens, const int64_t full_lens_strides[3],
+                                   const int32_t *part_ids, const int64_t part_ids_strides[4],
+                                   const int32_t *part_lens, const int64_t part_lens_strides[3],
+                                   const uint8_t *packed, const int64_t packed_strides[2], int B, int H, int Sq,
+                                   int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2, void *stream);
 
 #ifdef __cplusplus
 }

@@ -7,7 +7,7 @@ missing instead of falling back to anything in here.
 Two restatements of the reference algorithm live here:
 
 * ``sparse_oracle.c`` (built into ``liboracle.so`` by ``oracle/Makefile``), wrapped by
-  :func:`classify` and :func:`forward`;
+  :func:`classify`, :func:`forward` and :func:`pack_partial`;
 * the numpy functions :func:`classify_numpy` and :func:`forward_dense_fp64`, written a
   different way (per-tile popcount by reshape; dense fp64 softmax) so that the two can be
   checked against each other and against closed forms.
@@ -55,6 +55,8 @@ def _load():
     lib.oracle_forward.argtypes = (
         [f32p, f32p, f32p, f32p, u8p, i64p, i32p, i32p, i32p, i32p] + [ctypes.c_int] * 7 + [ctypes.c_float, ctypes.c_int]
     )
+    lib.oracle_pack_partial.restype = ctypes.c_int
+    lib.oracle_pack_partial.argtypes = [u8p, i64p] + [ctypes.c_int] * 6 + [i32p, i32p, u8p]
     lib.oracle_max_threads.restype = ctypes.c_int
     for fn in (lib.oracle_round_bf16, lib.oracle_round_fp16):
         fn.restype = ctypes.c_float
@@ -145,6 +147,30 @@ def classify_numpy(mask: np.ndarray, BQ: int, BK: int) -> OracleMetadata:
     fid, fl = compact(full)
     pid, pl = compact(part)
     return OracleMetadata(fid, fl, pid, pl)
+
+
+def pack_partial(mask: np.ndarray, BQ: int, BK: int, meta: OracleMetadata | None = None, fill: int = 0) -> np.ndarray:
+    """Bit-packed PARTIAL tiles, uint8 [B,H,nQ,nK,BQ*BK/8] (C loop ``oracle_pack_partial``).
+
+    Tile ``[b,h,qt,slot]`` holds the entries of KV tile ``meta.masked_kv_ids[b,h,qt,slot]``, rows first,
+    little-endian bits; slots past ``meta.masked_lens`` keep ``fill``.
+    """
+    lib = _load()
+    B, H, Sq, Sk = mask.shape
+    if Sq % BQ or Sk % BK or BK % 8:
+        raise ValueError("Sq % BLOCK_Q, Sk % BLOCK_K and BLOCK_K % 8 must be 0")
+    if meta is None:
+        meta = classify(mask, BQ, BK)
+    m8, strides = _mask_view(mask)
+    nQ, nK = Sq // BQ, Sk // BK
+    out = np.full((B, H, nQ, nK, BQ * BK // 8), fill, np.uint8)
+    ids_p = np.ascontiguousarray(meta.masked_kv_ids, dtype=np.int32)
+    len_p = np.ascontiguousarray(meta.masked_lens, dtype=np.int32)
+    rc = lib.oracle_pack_partial(_ptr(m8, ctypes.c_uint8), _ptr(strides, ctypes.c_int64), B, H, Sq, Sk, BQ, BK,
+                                 _ptr(ids_p, ctypes.c_int32), _ptr(len_p, ctypes.c_int32), _ptr(out, ctypes.c_uint8))
+    if rc != 0:
+        raise RuntimeError(f"oracle_pack_partial failed: {rc}")
+    return out
 
 
 def forward(q, k, v, mask, BQ: int, BK: int, meta: OracleMetadata | None = None, p_round: int = 0) -> np.ndarray:

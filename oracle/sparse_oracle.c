@@ -211,3 +211,39 @@ int oracle_forward(const float *q, const float *k, const float *v, float *out, c
     }
     return failed ? -2 : 0;
 }
+
+/*
+ * One bit per mask entry of every PARTIAL tile (the optional packed route of the HIP library; the reference
+ * has no such step: it re-reads the bool tile in every forward, sparse_attn_kernel.py:42-46).
+ *
+ * part_ids [B,H,nQ,nK] / part_lens [B,H,nQ] are the PARTIAL lists of oracle_classify.  out is
+ * [B,H,nQ,nK,BQ*BK/8] bytes, zero-filled by the caller: tile (qt, slot) holds the BQ x BK entries of KV tile
+ * part_ids[..., qt, slot], rows first, entry (r, c) in bit (c & 7) of byte (r*BK + c) >> 3; a byte != 0 in
+ * the mask sets the bit.  Slots >= the count stay as the caller left them.
+ * Pinned by tests/test_oracle_pack.py against numpy.packbits(bitorder="little") of the same tiles and
+ * against the closed form of the causal diagonal tiles.
+ */
+int oracle_pack_partial(const uint8_t *mask, const int64_t *ms, int B, int H, int Sq, int Sk, int BQ, int BK,
+                        const int32_t *part_ids, const int32_t *part_lens, uint8_t *out) {
+    if (BQ <= 0 || BK <= 0 || Sq % BQ || Sk % BK || BK % 8) return -1;
+    const int nQ = Sq / BQ, nK = Sk / BK;
+    const long tile_bytes = (long)BQ * BK / 8;
+    for (int b = 0; b < B; b++)
+        for (int h = 0; h < H; h++)
+            for (int i = 0; i < nQ; i++) {
+                const long row = ((long)b * H + h) * nQ + i;
+                for (int s = 0; s < part_lens[row]; s++) {
+                    const int j = part_ids[row * nK + s];
+                    uint8_t *tile = out + (row * nK + s) * tile_bytes;
+                    for (int r = 0; r < BQ; r++)
+                        for (int c = 0; c < BK; c++) {
+                            const uint8_t m = mask[(int64_t)b * ms[0] + (int64_t)h * ms[1] +
+                                                   (int64_t)(i * BQ + r) * ms[2] + (int64_t)(j * BK + c) * ms[3]];
+                            const long bit = (long)r * BK + c;
+                            if (m) tile[bit >> 3] |= (uint8_t)(1u << (bit & 7));
+                            else tile[bit >> 3] &= (uint8_t)~(1u << (bit & 7));
+                        }
+                }
+            }
+    return 0;
+}

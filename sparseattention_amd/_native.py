@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsparseattn_hip.so")
 
-SA_ABI_VERSION = 1
+SA_ABI_VERSION = 2
 SA_OK = 0
 SA_ERR_INVALID_ARGUMENT = -1
 SA_ERR_UNSUPPORTED = -2
@@ -27,6 +27,9 @@ EXPORTS = (
     "sa_mask_classify_workspace_bytes",
     "sa_mask_classify",
     "sa_sparse_attention_fwd",
+    "sa_mask_pack_partial_bytes",
+    "sa_mask_pack_partial",
+    "sa_sparse_attention_fwd_packed",
 )
 
 _lib = None
@@ -67,6 +70,14 @@ def load() -> ctypes.CDLL:
     lib.sa_sparse_attention_fwd.restype = ctypes.c_int
     lib.sa_sparse_attention_fwd.argtypes = (
         [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [ctypes.c_int] * 8 + [ctypes.c_float, _vp]
+    )
+    lib.sa_mask_pack_partial_bytes.restype = ctypes.c_size_t
+    lib.sa_mask_pack_partial_bytes.argtypes = [_i64p] + [ctypes.c_int] * 6
+    lib.sa_mask_pack_partial.restype = ctypes.c_int
+    lib.sa_mask_pack_partial.argtypes = [_vp, _i64p] + [ctypes.c_int] * 6 + [_vp, _i64p] * 3 + [_vp]
+    lib.sa_sparse_attention_fwd_packed.restype = ctypes.c_int
+    lib.sa_sparse_attention_fwd_packed.argtypes = (
+        [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [_vp, _i64p] + [ctypes.c_int] * 8 + [ctypes.c_float, _vp]
     )
     if lib.sa_abi_version() != SA_ABI_VERSION:
         raise RuntimeError(f"libsparseattn_hip ABI {lib.sa_abi_version()} != expected {SA_ABI_VERSION}")

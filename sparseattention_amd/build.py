@@ -17,7 +17,12 @@ CSRC = os.path.join(_HERE, "csrc")
 INCLUDE = os.path.join(_ROOT, "include")
 LIB_PATH = os.path.join(_HERE, "libsparseattn_hip.so")
 
-SOURCES = ["sparseattn_api.hip", "mask_classify.hip", "sparse_fwd.hip"]
+# (source, object name, extra defines).  The forward kernels are one source compiled per element type and
+# mask source, so that the variants build in parallel.
+UNITS = [("sparseattn_api.hip", "sparseattn_api.o", []), ("mask_classify.hip", "mask_classify.o", []),
+         ("sparse_fwd.hip", "sparse_fwd.o", [])]
+UNITS += [("sparse_fwd_inst.hip", f"sparse_fwd_dt{dt}_pk{pk}.o", [f"-DSA_FWD_DT={dt}", f"-DSA_FWD_PK={pk}"])
+          for dt in (0, 1) for pk in (0, 1)]
 
 # -packed-fp32-ops is switched off on purpose: the compiler must not form v_pk_*_f32 from float code.
 HIPCC_FLAGS = [
@@ -57,12 +62,13 @@ def build_library(verbose: bool = False, extra_flags=()) -> str:
     hipcc = _hipcc()
     obj_dir = os.path.join(_HERE, "build")
     os.makedirs(obj_dir, exist_ok=True)
-    objs = [os.path.join(obj_dir, s.replace(".hip", ".o")) for s in SOURCES]
-    cmds = [[hipcc, *HIPCC_FLAGS, *extra_flags, "-c", os.path.join(CSRC, s), "-o", o] for s, o in zip(SOURCES, objs)]
+    objs = [os.path.join(obj_dir, o) for _, o, _ in UNITS]
+    cmds = [[hipcc, *HIPCC_FLAGS, *extra_flags, *defs, "-c", os.path.join(CSRC, src), "-o", obj]
+            for (src, _, defs), obj in zip(UNITS, objs)]
     if verbose:
         for c in cmds:
             print(" ".join(c))
-    with ThreadPoolExecutor(max_workers=min(4, len(cmds))) as ex:
+    with ThreadPoolExecutor(max_workers=min(os.cpu_count() or 4, len(cmds), 8)) as ex:
         list(ex.map(_run, cmds))
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", LIB_PATH])
     return LIB_PATH

@@ -25,8 +25,24 @@ struct CompactParams {
     int64_t fis[4], fls[3], pis[4], pls[3];  // output strides in elements
 };
 
+// Bit-packing of the PARTIAL tiles: tile (qt, slot) of a distinct plane is the slot-th entry of that Q tile's
+// PARTIAL list; its BQ x BK mask entries become BQ*BK/8 bytes, row-major, entry (r, c) in bit (c & 7) of byte
+// (r*BK + c) >> 3.
+struct PackParams {
+    const uint8_t *mask;
+    int64_t sb, sh, sq, sk;  // mask strides in bytes over the distinct planes
+    const int32_t *part_ids, *part_lens;
+    int64_t pis[4], pls[3];  // list strides in elements, indexed with the distinct-plane coordinates
+    uint8_t *packed;
+    int64_t ob, oh;  // bytes between the packed planes along b and h
+    int uB, uH;
+    int BQ, BK, nQ, nK;
+    int vec8;  // 1: key stride 1 and every row segment 8-byte aligned, so 8 entries load as one qword
+};
+
 hipError_t launch_classify(const ClassifyParams &p, bool wide, hipStream_t stream);
 hipError_t launch_compact(const CompactParams &p, hipStream_t stream);
+hipError_t launch_pack(const PackParams &p, hipStream_t stream);
 
 // ---- block-sparse forward ------------------------------------------------------------------------
 struct FwdParams {
@@ -40,6 +56,10 @@ struct FwdParams {
     int B, H, Sq, Sk, nQ;
     int BK, lbk;    // KV tile width and its log2
     int mask_vec4;  // 1: mask columns are contiguous and 4-byte aligned, so 4 entries load as one dword
+    // Bit-packed PARTIAL tiles (PackParams layout), or null: then the mask itself is read.
+    const uint8_t *packed;
+    int64_t pks[2];  // bytes between packed planes along b and h (0 where the mask is broadcast)
+    int nK;          // KV tiles per row of tiles (slots per Q tile in `packed`)
     float scale;    // softmax scale / ln 2
 };
 

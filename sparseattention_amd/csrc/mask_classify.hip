@@ -10,6 +10,9 @@
 //   compact_kernel
 //       one wave per (b, h, Q tile): ballot + popcount prefix over the class bytes, writing the two
 //       ascending index lists and their counts (mask_utils.py:72-82).
+//   pack_partial_kernel (optional, no counterpart in the reference)
+//       one bit per entry of every PARTIAL tile, so that the forward reads BQ*BK/8 contiguous bytes per
+//       partial tile instead of BQ row segments of the mask (sparse_attn_kernel.py:42-46).
 //
 // A byte != 0 counts as "attend", so masks that were viewed from uint8 storage behave like torch.sum.
 #include <hip/hip_runtime.h>
@@ -139,7 +142,53 @@ __global__ __launch_bounds__(256) void compact_kernel(const CompactParams p) {
     }
 }
 
+// grid (slot lanes, nQ, distinct planes), 256 threads.  Workgroup x takes the PARTIAL slots x, x + gridDim.x, ...
+// of its Q tile; a thread makes one output byte at a time from 8 neighbouring mask entries of one row.
+__global__ __launch_bounds__(256) void pack_partial_kernel(const PackParams p) {
+    const int qt = blockIdx.y;
+    const int plane = blockIdx.z;
+    const int ub = plane / p.uH, uh = plane - ub * p.uH;
+    const int len = p.part_lens[ub * p.pls[0] + uh * p.pls[1] + qt * p.pls[2]];
+    const int32_t *ids = p.part_ids + ub * p.pis[0] + uh * p.pis[1] + qt * p.pis[2];
+    const int bpr = p.BK >> 3;                 // output bytes per tile row
+    const int tile_bytes = p.BQ * bpr;
+    const uint8_t *rows = p.mask + (int64_t)ub * p.sb + (int64_t)uh * p.sh + (int64_t)qt * p.BQ * p.sq;
+    uint8_t *out_q = p.packed + (int64_t)ub * p.ob + (int64_t)uh * p.oh + (int64_t)qt * p.nK * tile_bytes;
+    for (int slot = blockIdx.x; slot < len; slot += gridDim.x) {
+        const int64_t col0 = (int64_t)ids[(int64_t)slot * p.pis[3]] * p.BK;
+        uint8_t *out = out_q + (int64_t)slot * tile_bytes;
+        for (int o = threadIdx.x; o < tile_bytes; o += 256) {
+            const int r = o / bpr, cb = o - r * bpr;
+            const uint8_t *src = rows + (int64_t)r * p.sq + (col0 + 8 * cb) * p.sk;
+            uint32_t lo, hi;
+            if (p.vec8) {
+                const uint2 w = *(const uint2 *)src;
+                lo = w.x;
+                hi = w.y;
+            } else {
+                lo = hi = 0u;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    lo |= (uint32_t)src[(int64_t)i * p.sk] << (8 * i);
+                    hi |= (uint32_t)src[(int64_t)(4 + i) * p.sk] << (8 * i);
+                }
+            }
+            // 0x80 per non-zero byte -> one bit per byte, entry i of the group in bit i
+            const uint32_t a = nonzero_bytes(lo) >> 7, b = nonzero_bytes(hi) >> 7;
+            // (bits 0, 8, 16, 24 times 2^21 + 2^14 + 2^7 + 1 meet in bits 21..24, without carries)
+            const uint32_t nib_lo = ((a * 0x00204081u) >> 21) & 0xfu, nib_hi = ((b * 0x00204081u) >> 21) & 0xfu;
+            out[o] = (uint8_t)(nib_lo | (nib_hi << 4));
+        }
+    }
+}
+
 }  // namespace
+
+hipError_t launch_pack(const PackParams &p, hipStream_t stream) {
+    const int lanes = p.nK < 8 ? p.nK : 8;
+    hipLaunchKernelGGL(pack_partial_kernel, dim3(lanes, p.nQ, p.uB * p.uH), dim3(256), 0, stream, p);
+    return hipGetLastError();
+}
 
 hipError_t launch_classify(const ClassifyParams &p, bool wide, hipStream_t stream) {
     if (wide) {

@@ -1,668 +1,20 @@
-// Block-sparse flash-attention forward for gfx950 (MI355X).
-//
-// Replaces the Triton kernels sparse_attention_kernel / _sparse_inner
-// (sparseattention/sparse_attn_kernel.py:74-146 and :10-63).
-//
-// Work decomposition
-//   One workgroup per (Q tile of BQ rows, b, h); NW = BQ/32 waves, wave w owns query rows
-//   [32w, 32w+32) of the tile.  The listed KV tiles of that Q tile (all FULL tiles, then all PARTIAL
-//   tiles, as the reference orders them) form one stream that is consumed in chunks of 64 key rows:
-//   BK=16 -> 4 list entries per chunk, BK=32 -> 2, BK>=64 -> BK/64 chunks per entry.  Softmax is
-//   row-wise, so gathered tiles that are not neighbours in K can share a chunk.
-//
-// Register layout (v_mfma_f32_32x32x16_{bf16,f16}; lane = 32*hh + l32)
-//   S^T = K . Q^T   A = K rows (kv = l32 of each 32-row block), B = Q^T (q = l32), contraction over d;
-//                   the result leaves lane (l32, hh) holding query l32 and keys 8g+4hh+j
-//                   (g,j in 0..3, register 4g+j) of each 32-key block.  Every lane owns one query
-//                   row, so row max / row sum are in-lane reductions plus one exchange with lane^32.
-//   O^T = V^T . P^T A = V^T (d = l32 of each 32-wide block), B = P^T (q = l32), contraction over keys.
-//                   Registers 8c..8c+7 of a S^T block are exactly the B operand of the c-th
-//                   16-key MFMA step, so P never leaves registers; the matching A operand is read
-//                   from row-major V in LDS with the transposing ds_read_b64_tr_b16.
-//
-// LDS: two buffers each for K and V (64 rows per buffer), filled straight from global memory
-// (global_load_lds_dwordx4, 1 KiB per wave instruction) one chunk ahead of the MFMAs.  Rows are
-// unpadded; bank conflicts are avoided by XOR-swizzling the 16-byte pieces of a row (k_swizzle,
-// v_swizzle).
-#include "fwd_common.h"
+// Dispatch of the block-sparse forward to the translation unit that holds the kernels for the element type
+// and for the source of the PARTIAL tiles' mask entries (see sparse_fwd_inst.hip).
+#include "kernels.h"
 
 namespace sa {
 
-namespace {
-
-template <int N, class F>
-__device__ __forceinline__ void static_for(F &&f) {  // f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)
-    if constexpr (N > 0) {
-        static_for<N - 1>(f);
-        f(std::integral_constant<int, N - 1>{});
-    }
-}
-
-// "At most n vector-memory operations of this wave still in flight", n a small run-time value.
-__device__ __forceinline__ void wait_vm_at_most(int n, int step) {
-    if (n <= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    else if (n == 1) {
-        if (step == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-        else if (step == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-        else if (step == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    } else {
-        if (step == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-        else if (step == 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-        else if (step == 8) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-}
-
-// MODE 0: BK = 16, MODE 1: BK = 32, MODE 2: BK >= 64 (runtime log2 in p.lbk).
-// NS: LDS stages per operand (2 or 4); chunks are fetched NS-1 ahead of the one being computed.
-// PP: the two waves that share a SIMD (w and w+4 of an 8-wave workgroup) run half a chunk apart, one in its
-// S phase while the other is in its P.V phase (see the main loop).
-template <int DT, int D, int NW, int MODE, int NS, bool PP>
-__global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(const FwdParams p) {
-    using E = Elem<DT>;
-    constexpr int ROWB = D * 2;                   // bytes per K/V row in LDS
-    constexpr int KBUF = 64 * ROWB, VBUF = 64 * ROWB;
-    constexpr int RPI = 1024 / ROWB;              // rows written by one wave-wide direct load (1 KiB)
-    constexpr int NLD = 64 / (RPI * NW);          // direct loads per wave per chunk, each for K and for V
-    constexpr int PPR = ROWB / 16;                // 16-byte pieces per row
-    constexpr int EPC = MODE == 0 ? 4 : (MODE == 1 ? 2 : 1);  // list entries per chunk
-    constexpr int LBKC = MODE == 0 ? 4 : 5;                   // log2(BK) when MODE < 2
-    static_assert(64 % (RPI * NW) == 0, "staging layout");
-
-    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-    static_assert(NS == 2 || NS == 4, "stage count");
-    constexpr int PD = NS - 1;  // fetch distance in chunks
-    // [K stage 0..NS-1][V stage 0..NS-1][first key column of every list entry, kListCap ints]
-    int *const ent = reinterpret_cast<int *>(smem + NS * KBUF + NS * VBUF);
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int l32 = lane & 31, hh = lane >> 5;
-
-    // Workgroup -> (b, h, Q tile).  Hardware hands consecutive workgroup ids to the 8 XCDs in turn; the
-    // remap gives each XCD a contiguous range of the (b,h)-major order so that the Q tiles sharing one
-    // K/V plane run on the XCD whose L2 already holds it.  Planes are taken two at a time with their Q tiles
-    // interleaved, last Q tile first (under causal-like masks it has the longest list): the slots that finish
-    // the short tiles of one pair then pick up the long tiles of the next, which evens out the load.
-    const int total = gridDim.x, per = total >> 3;
-    int lin = blockIdx.x;
-    if (lin < (per << 3)) lin = (lin & 7) * per + (lin >> 3);
-    const int pair = lin / (2 * p.nQ), r = lin - pair * 2 * p.nQ;
-    const bool paired = 2 * pair + 1 < p.B * p.H;  // the last plane of an odd count goes alone
-    const int bh = 2 * pair + (paired ? (r & 1) : 0);
-    const int qt = p.nQ - 1 - (paired ? (r >> 1) : r);
-    const int b = bh / p.H, h = bh - b * p.H;
-
-    const uint16_t *kbase = p.k + b * p.ks[0] + h * p.ks[1];
-    const uint16_t *vbase = p.v + b * p.vs[0] + h * p.vs[1];
-    const int qrow = qt * (NW * 32) + wave * 32 + l32;  // the query row this lane owns
-    const uint8_t *mrow = p.mask + b * p.ms[0] + h * p.ms[1] + (int64_t)qrow * p.ms[2];
-
-    const int32_t *fid = p.full_ids + b * p.fis[0] + h * p.fis[1] + qt * p.fis[2];
-    const int32_t *pid = p.part_ids + b * p.pis[0] + h * p.pis[1] + qt * p.pis[2];
-    const int F = p.full_lens[b * p.fls[0] + h * p.fls[1] + qt * p.fls[2]];
-    const int P = p.part_lens[b * p.pls[0] + h * p.pls[1] + qt * p.pls[2]];
-    const int NE = F + P;
-    const int T = MODE == 2 ? (NE << (p.lbk - 6)) : ((NE + EPC - 1) / EPC);
-
-    // Q^T operand: lane (l32, hh) keeps d = 16c + 8hh .. +7 of its query row for every 16-wide step c.
-    u32x4 qf[D / 16];
-    {
-        const uint16_t *qp = p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2] + 8 * hh;
-#pragma unroll
-        for (int c = 0; c < D / 16; c++) qf[c] = *(const u32x4 *)(qp + 16 * c);
-        // The scale (softmax scale / ln 2) goes into Q once, so that the S MFMAs deliver exp2 arguments.
-#pragma unroll
-        for (int c = 0; c < D / 16; c++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) qf[c][e] = E::scale2(qf[c][e], p.scale);
-    }
-
-    // Online-softmax state of this lane's query row.  Exponentials are taken against a reference value m_ref
-    // (exp2 units).  The S MFMAs start from the accumulator -m_ref (neg_m: the same value in all 16 registers,
-    // one query per lane), so a score leaves the matrix unit as the exp2 argument itself.  raise_above is the
-    // largest such argument tolerated before m_ref moves: kMaxSlack, or "anything finite" until the row has
-    // seen its first attended key.
-    float m_ref = 0.f;
-    float raise_above = -3.0e38f;
-    f32x16 neg_m;
-#pragma unroll
-    for (int i = 0; i < 16; i++) neg_m[i] = 0.f;
-    // Running row sums of P, kept by a 16x16x32 MFMA whose B operand is P itself.  In that instruction lane l
-    // supplies column l%16 and key group l/16, so the P registers of query rows r and r+16 land in the same
-    // column; the A operand separates them again: its row i is all ones over the key groups of parity i&1 and
-    // zero elsewhere.  Result register 0 of lane l is then the row sum of query l%16 and register 1 that of
-    // query l%16 + 16; a lane reads the one that belongs to its own row.
-    f32x4 acc_l = {0.f, 0.f, 0.f, 0.f};
-    const uint32_t sel1 = (((lane >> 4) ^ lane) & 1) == 0 ? E::ones4().x : 0u;
-    const u32x4 sum_sel = {sel1, sel1, sel1, sel1};
-    f32x16 acc[D / 32];
-#pragma unroll
-    for (int db = 0; db < D / 32; db++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) acc[db][i] = 0.f;
-
-    // ---- per-lane LDS offsets (bytes, relative to the start of a K or V buffer) -------------------
-    // K operand of step c: row 32kb + l32, piece 2c + hh, swizzled.  (2c + hh) ^ s == (2c) ^ (hh ^ s).
-    int koff[D / 16];
-    {
-        const int t = hh ^ k_swizzle<D>(l32);
-#pragma unroll
-        for (int c = 0; c < D / 16; c++) koff[c] = l32 * ROWB + 16 * ((2 * c) ^ t);
-    }
-    // V^T operand (transposing read): within each 16-lane group, lane t supplies the address of 4
-    // consecutive d of key row (t >> 2) and receives the 4 key rows of d column t.
-    int voff[D / 32];
-    {
-        const int tr_row = 4 * hh + ((lane & 15) >> 2);        // + 16kc (+8 for the second read)
-        const int x = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);  // piece within the 32-wide d block
-        const int sw = v_swizzle<D>(tr_row) >> 2;               // 16kc and 8 leave the swizzle bits alone
-#pragma unroll
-        for (int db = 0; db < D / 32; db++) voff[db] = tr_row * ROWB + 64 * (db ^ sw) + 16 * x + 8 * (lane & 1);
-    }
-    // Direct-load staging: load i of this wave fills rows [RPI*(NW*i + wave), +RPI) of the chunk; lane
-    // writes row ld_row(i), LDS piece lane % PPR, and therefore fetches the swizzled source piece.
-    // The source address splits into a wave-uniform part (plane base + first row of the list entry, scalar
-    // arithmetic per chunk) and a per-lane byte offset that never changes (row within the entry, swizzled
-    // piece), so staging a chunk costs no vector arithmetic.
-    const int ld_r0 = lane / PPR, ld_slot = lane % PPR;
-    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const SA_LDS uint8_t *)smem);
-    uint32_t ld_koff[NLD], ld_voff[NLD];
-#pragma unroll
-    for (int i = 0; i < NLD; i++) {
-        const int r = RPI * (NW * i + wave_u) + ld_r0;
-        const int within = MODE == 2 ? r : (r & ((1 << LBKC) - 1));
-        ld_koff[i] = (uint32_t)((within * p.ks[2] + 8 * (ld_slot ^ k_swizzle<D>(r))) * 2);
-        ld_voff[i] = (uint32_t)((within * p.vs[2] + 8 * (ld_slot ^ v_swizzle<D>(r))) * 2);
-    }
-
-    // The Q tile's list (FULL entries, then PARTIAL entries) as first key columns, copied to LDS once:
-    // loads issued after the first barrier cannot use the scalar cache, and a vector load of an index in
-    // front of every chunk would put a full memory round trip on the critical path.
-    const bool list_in_lds = NE <= kListCap;
-    if (list_in_lds) {
-        for (int e = tid; e < NE; e += NW * 64) {
-            const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
-            ent[e] = MODE == 2 ? (idx << p.lbk) : (idx << LBKC);
-        }
-    }
-    // First key column of every list entry in chunk t (t < T), plus which entries exist / are partial, in two
-    // steps: entries_read issues the reads of the list (the values are the same in all lanes), entries_use turns
-    // them into scalars.  The main loop reads the entries of a chunk one iteration before it needs them, so
-    // that no wave waits for the list.
-    auto entry_read = [&](int e) -> int {
-        if (list_in_lds) return ent[e];
-        const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
-        return MODE == 2 ? (idx << p.lbk) : (idx << LBKC);
-    };
-    auto entries_read = [&](int t, int(&raw)[EPC]) {
-        if constexpr (MODE == 2) {
-            raw[0] = entry_read(t >> (p.lbk - 6));
-        } else {
-#pragma unroll
-            for (int j = 0; j < EPC; j++) {
-                const int e = t * EPC + j;
-                raw[j] = entry_read(e < NE ? e : t * EPC);  // absent entries re-read the chunk's first one;
-            }                                                // their scores are discarded
-        }
-    };
-    auto entries_use = [&](int t, const int(&raw)[EPC], int(&col)[EPC], unsigned &valid, unsigned &part) {
-        valid = 0u;
-        part = 0u;
-        if constexpr (MODE == 2) {
-            const int sh = p.lbk - 6;
-            const int e = t >> sh, sub = t & ((1 << sh) - 1);
-            col[0] = __builtin_amdgcn_readfirstlane(raw[0]) + (sub << 6);
-            valid = 1u;
-            part = e >= F ? 1u : 0u;
-        } else {
-#pragma unroll
-            for (int j = 0; j < EPC; j++) {
-                const int e = t * EPC + j;
-                col[j] = __builtin_amdgcn_readfirstlane(raw[j]);
-                if (e < NE) {
-                    valid |= 1u << j;
-                    if (e >= F) part |= 1u << j;
-                }
-            }
-        }
-    };
-    auto chunk_entries = [&](int t, int(&col)[EPC], unsigned &valid, unsigned &part) {
-        int raw[EPC];
-        entries_read(t, raw);
-        entries_use(t, raw, col, valid, part);
-    };
-
-    // Global -> LDS for one chunk, without passing through registers: 2*NLD direct loads per wave (piece 2i is
-    // load i of K, piece 2i+1 load i of V).  A wave that issues them back to back sits at the issue stage until
-    // the address unit has taken them all, while every other wave of the CU does the same; the main loop
-    // therefore hands them out one at a time between the MFMA bundles of the chunk being computed.
-    struct StagePlan {
-        const uint16_t *kp[EPC], *vp[EPC];  // first row of every list entry of the chunk (scalar registers)
-    };
-    auto plan_chunk = [&](const int(&col)[EPC], StagePlan &pl) {
-#pragma unroll
-        for (int j = 0; j < EPC; j++) {
-            pl.kp[j] = kbase + (int64_t)col[j] * p.ks[2];
-            pl.vp[j] = vbase + (int64_t)col[j] * p.vs[2];
-        }
-    };
-    auto stage_piece = [&](int buf, int piece, const StagePlan &pl) {
-        const int i = piece >> 1;
-        // rows [rbase, rbase + RPI) lie inside one list entry; when the rows of all waves of load i do, the
-        // entry is known at compile time
-        constexpr bool kEntryByLoad = MODE == 2 || RPI * NW <= (1 << LBKC);
-        const int rbase = RPI * (NW * i + wave_u);
-        const uint16_t *ks_ = pl.kp[0], *vs_ = pl.vp[0];
-        if constexpr (MODE != 2) {
-            const int j = kEntryByLoad ? ((RPI * NW * i) >> LBKC) : (rbase >> LBKC);
-#pragma unroll
-            for (int jj = 1; jj < EPC; jj++)
-                if (j == jj) {
-                    ks_ = pl.kp[jj];
-                    vs_ = pl.vp[jj];
-                }
-        }
-        if ((piece & 1) == 0) dma16(ks_, ld_koff[i], lds0 + buf * KBUF + rbase * ROWB);
-        else dma16(vs_, ld_voff[i], lds0 + NS * KBUF + buf * VBUF + rbase * ROWB);
-    };
-    auto stage_chunk = [&](int buf, const int(&col)[EPC]) {  // all pieces at once (prologue)
-        StagePlan pl;
-        plan_chunk(col, pl);
-#pragma unroll
-        for (int i = 0; i < 2 * NLD; i++) stage_piece(buf, i, pl);
-    };
-
-    // Mask bytes of this lane's eight 4-key groups in a chunk (non-zero byte = attended key).  Called for
-    // chunks with a PARTIAL or absent entry only.  FULL entries are read too (their bytes are all set);
-    // absent entries re-read the chunk's first entry and are discarded when the mask is applied.
-    // No branches, eight independent loads, and no use of the loaded values here.
-    auto load_mask = [&](const int(&col)[EPC], uint32_t(&mk)[2][4]) {
-        int64_t c[2][4];
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                int j, within;
-                if constexpr (MODE == 0) {
-                    j = 2 * kb + (g >> 1);
-                    within = 8 * (g & 1) + 4 * hh;
-                } else if constexpr (MODE == 1) {
-                    j = kb;
-                    within = 8 * g + 4 * hh;
-                } else {
-                    j = 0;
-                    within = 32 * kb + 8 * g + 4 * hh;
-                }
-                c[kb][g] = col[j] + within;
-            }
-        if (p.mask_vec4) {
-#pragma unroll
-            for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-                for (int g = 0; g < 4; g++) mk[kb][g] = *(const uint32_t *)(mrow + c[kb][g]);
-        } else {
-#pragma unroll
-            for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const uint8_t *m0 = mrow + c[kb][g] * p.ms[3];
-                    mk[kb][g] = (uint32_t)m0[0] | ((uint32_t)m0[p.ms[3]] << 8) | ((uint32_t)m0[2 * p.ms[3]] << 16) |
-                                ((uint32_t)m0[3 * p.ms[3]] << 24);
-                }
-        }
-    };
-
-    // One chunk from stage BUF, in two phases.
-    // S phase: s = K . Q^T - m_ref.  When `fetch`, the pieces of the chunk planned in `pl` are sent to stage
-    // FBUF between its MFMA bundles.
-    auto phase_s = [&](auto buf_c, f32x16(&s)[2], auto fbuf_c, bool fetch, const StagePlan &pl) {
-        constexpr int BUF = decltype(buf_c)::value;
-        constexpr int FBUF = decltype(fbuf_c)::value;
-        const uint8_t *kb_ = smem + BUF * KBUF;
-
-        // S^T = K . Q^T in bundles of two MFMAs (the two key blocks of d step c), operand reads kPfS bundles
-        // ahead.  Within a bundle the MFMA that uses the younger read goes first, so one wait covers both.
-        constexpr int NC = D / 16;
-        constexpr int kPfS = 3;
-        u32x4 kf0[NC], kf1[NC];
-        auto k_read = [&](int c) {
-            kf0[c] = *(const u32x4 *)(kb_ + koff[c]);
-            kf1[c] = *(const u32x4 *)(kb_ + 32 * ROWB + koff[c]);
-        };
-#pragma unroll
-        for (int c = 0; c < kPfS; c++) k_read(c);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int c = 0; c < NC; c++) {
-            s[1] = E::mfma(kf1[c], qf[c], c == 0 ? neg_m : s[1]);
-            s[0] = E::mfma(kf0[c], qf[c], c == 0 ? neg_m : s[0]);
-            if (c + kPfS < NC) k_read(c + kPfS);
-            if (fetch) {
-#pragma unroll
-                for (int i = 2 * NLD * c / NC; i < 2 * NLD * (c + 1) / NC; i++) stage_piece(FBUF, i, pl);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-    // P.V phase: mask, online softmax, O^T += V^T . P^T.  between(b, NB) is called once per MFMA bundle b of NB;
-    // the main loop uses it to spread scalar bookkeeping over the phase, where it hides behind the MFMAs.
-    auto phase_pv = [&](auto buf_c, f32x16(&s)[2], bool special, unsigned valid, const uint32_t(&mk)[2][4],
-                        auto &&between) {
-        constexpr int BUF = decltype(buf_c)::value;
-        const uint8_t *vb_ = smem + NS * KBUF + BUF * VBUF;
-        if (special) {
-#pragma unroll
-            for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const int j = MODE == 0 ? 2 * kb + (g >> 1) : (MODE == 1 ? kb : 0);  // list entry of this group
-                    const uint32_t w = ((valid >> j) & 1u) ? mk[kb][g] : 0u;
-#pragma unroll
-                    for (int jj = 0; jj < 4; jj++)
-                        if (((w >> (8 * jj)) & 0xffu) == 0u) s[kb][4 * g + jj] = kNegInf;
-                }
-        }
-
-        // Online softmax in exp2 units (sparse_attn_kernel.py:47-58), with a lagging reference value: s holds
-        // score*scale - m_ref.  Only when some row's largest argument exceeds raise_above does m_ref move.
-        float mx = kNegInf;
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[kb][i]);
-        mx = half_swap_max(mx);
-        const bool raise = mx > raise_above;  // false for rows without an attended key so far (mx = -inf)
-        if (__builtin_amdgcn_ballot_w64(raise) != 0ull) {
-            // rows that raise: m_ref += mx, the arguments drop by mx, what was accumulated shrinks by 2^-mx
-            // (nothing was accumulated if this is the row's first attended key: factor 0, not 2^-mx, which
-            // may be infinite)
-            const float delta = raise ? mx : 0.f;
-            const float a = raise ? (raise_above == kMaxSlack ? __builtin_amdgcn_exp2f(-mx) : 0.f) : 1.f;
-            m_ref += delta;
-            raise_above = raise ? kMaxSlack : raise_above;
-#pragma unroll
-            for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) s[kb][i] -= delta;
-#pragma unroll
-            for (int i = 0; i < 16; i++) neg_m[i] = -m_ref;
-#pragma unroll
-            for (int i = 0; i < 2; i++) acc_l[i] *= a;  // the lane only ever reads the one of its own row
-#pragma unroll
-            for (int db = 0; db < D / 32; db++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) acc[db][i] *= a;
-        }
-
-        // P = exp2(s), rounded to the input dtype, and O^T += V^T . P^T.
-        // MFMA (key step kc, d block db) needs only the kc-th group of 8 P values, so the loop is a software
-        // pipeline of bundles pinned by scheduling barriers: two MFMAs (d blocks 2h, 2h+1 of one key step) |
-        // the transposing reads for a later bundle | half of the next key step's exponentials.
-        // The row sum comes from one small MFMA per key step (see acc_l): it adds up the 16 keys of the step,
-        // both lane halves included, and it adds up the ROUNDED values, the ones that enter P.V, so the output
-        // is an exact convex combination of value rows (the reference sums the unrounded ones; the difference
-        // is bounded by the rounding of P).
-        constexpr int NDB = D / 32;
-        constexpr int NB = 4 * NDB / 2;  // bundles; bundle b: key step b / (NDB/2), d blocks 2*(b % (NDB/2)) + {0,1}
-        constexpr int BPK = NDB / 2;     // bundles per key step
-        constexpr int kPfV = 2;
-        constexpr int PER = 8 / BPK;     // P values of the next key step produced per bundle
-        uint32_t pw[16];                 // P, two keys per dword, in MFMA operand order
-        auto p_values = [&](int kc, int first, int count) {
-#pragma unroll
-            for (int i = first; i < first + count; i += 2) {
-                const float x0 = __builtin_amdgcn_exp2f(s[kc >> 1][8 * (kc & 1) + i]);
-                const float x1 = __builtin_amdgcn_exp2f(s[kc >> 1][8 * (kc & 1) + i + 1]);
-                pw[4 * kc + (i >> 1)] = E::pack2(x0, x1);
-            }
-        };
-        u32x2 vlo[2 * NB], vhi[2 * NB];
-        auto v_read = [&](int b) {
-#pragma unroll
-            for (int u = 0; u < 2; u++) {
-                const int kc = b / BPK, db = 2 * (b % BPK) + u;
-                const uint8_t *vp = vb_ + 16 * kc * ROWB + voff[db];
-                vlo[2 * b + u] = E::tr_read(vp);
-                vhi[2 * b + u] = E::tr_read(vp + 8 * ROWB);
-            }
-        };
-#pragma unroll
-        for (int b = 0; b < kPfV; b++) v_read(b);
-        p_values(0, 0, 8);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int b = 0; b < NB; b++) {
-            const int kc = b / BPK;
-            const u32x4 pk4 = u32x4{pw[4 * kc], pw[4 * kc + 1], pw[4 * kc + 2], pw[4 * kc + 3]};
-#pragma unroll
-            for (int u = 1; u >= 0; u--) {
-                const int db = 2 * (b % BPK) + u, i = 2 * b + u;
-                acc[db] = E::mfma(u32x4{vlo[i].x, vlo[i].y, vhi[i].x, vhi[i].y}, pk4, acc[db]);
-            }
-            if (b % BPK == BPK - 1) acc_l = E::mfma16(sum_sel, pk4, acc_l);
-            if (b + kPfV < NB) v_read(b + kPfV);
-            if (kc + 1 < 4) p_values(kc + 1, PER * (b % BPK), PER);
-            between(b, NB);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-
-    // Makes the compiler account for a completed vector-memory load here (it emits its own wait, which
-    // costs nothing once the data has landed) instead of in front of a later use, where the wait would
-    // also cover direct loads it does not know about.
-    auto settle = [](const uint32_t(&mk)[2][4]) {
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) asm volatile("" ::"v"(mk[kb][g]));
-    };
-
-    if constexpr (PP) {
-        // Ping-pong schedule.  Every wave runs  barrier | S phase | barrier | P.V phase  per chunk; waves 4..7
-        // enter the sequence one barrier later than waves 0..3, so between two barriers one wave of each SIMD
-        // issues the MFMA-only S phase while the other does softmax and P.V, and the matrix unit always has a
-        // taker.  Chunk t is needed first by waves 0..3 after barrier 2t and last by waves 4..7 before barrier
-        // 2t+3; it is fetched two chunks ahead into a ring of 4 stages, whose slot was given up before barrier
-        // 2t-1.  Before arriving at barrier 2t every wave has waited for its own pieces of chunk t.
-        static_assert(!PP || (NW == 8 && NS == 4), "ping-pong layout");
-        if (T > 0) {
-            const int late = wave_u >> 2;  // 1: this wave runs half a chunk behind
-            int col[EPC], coln[EPC];       // entries of the chunk at hand / of the next chunk to look at
-            unsigned valid, part, validn = 0u, partn = 0u;
-            uint32_t mk[2][2][4] = {};
-            bool sp[2] = {false, false};
-            unsigned vl[2] = {0u, 0u};
-            constexpr unsigned ALL = (1u << EPC) - 1u;
-            constexpr int kOpsPerChunk = 2 * NLD;
-            __syncthreads();  // the list in LDS is complete
-            chunk_entries(0, col, valid, part);
-            stage_chunk(0, col);
-            sp[0] = part != 0u || valid != ALL;
-            vl[0] = valid;
-            if (sp[0]) load_mask(col, mk[0]);
-#pragma unroll
-            for (int j = 0; j < EPC; j++) coln[j] = col[j];
-            if (1 < T) {
-                chunk_entries(1, coln, validn, partn);
-                stage_chunk(1, coln);
-            }
-#pragma unroll
-            for (int c = 0; c < D / 16; c++) asm volatile("" ::"v"(qf[c]));
-            int raw[EPC] = {};  // list entries of the chunk after next, read ahead
-            if (2 < T) entries_read(2, raw);
-            if (sp[0]) settle(mk[0]);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __syncthreads();
-            if (late) __syncthreads();
-            for (int t = 0; t < T; t += NS) {
-                static_for<NS>([&](auto jc) {
-                    constexpr int j = decltype(jc)::value;
-                    constexpr int cur = j & 1, nxt = cur ^ 1;
-                    const int tc = t + j;
-                    if (tc < T) {
-                        // own pieces of chunk tc have landed; chunk tc+1 may be in flight
-                        wait_vm_at_most((tc + 1 < T ? tc + 1 : T - 1) - tc, kOpsPerChunk);
-                        if (sp[cur]) settle(mk[cur]);
-                        __syncthreads();
-                        sp[nxt] = false;
-                        if (tc + 1 < T) {  // coln: entries of chunk tc+1
-                            sp[nxt] = partn != 0u || validn != ALL;
-                            vl[nxt] = validn;
-                            if (sp[nxt]) load_mask(coln, mk[nxt]);
-                        }
-                        const bool fetch = tc + 2 < T;
-                        if (fetch) {
-                            entries_use(tc + 2, raw, coln, validn, partn);
-                            if (tc + 3 < T) entries_read(tc + 3, raw);
-                        }
-                        StagePlan pl;
-                        plan_chunk(coln, pl);
-                        f32x16 s[2];
-                        phase_s(jc, s, std::integral_constant<int, (j + 2) % NS>{}, fetch, pl);
-                        // own pieces of chunk tc+1 have landed; chunk tc+2 may be in flight
-                        wait_vm_at_most((tc + 2 < T ? tc + 2 : T - 1) - (tc + 1), kOpsPerChunk);
-                        __syncthreads();
-                        phase_pv(jc, s, sp[cur], vl[cur], mk[cur], [](int, int) {});
-                    }
-                });
-            }
-            if (!late) __syncthreads();
-        }
-    } else if (T > 0) {
-        static_assert(PP || NS == 2, "two stages: the chunk being computed and the one being fetched");
-        int col[EPC], coln[EPC];  // entries of chunk 0 / of the chunk that the current iteration fetches
-        unsigned valid, part;
-        uint32_t mk[2][2][4] = {};  // mask words of the chunk being computed / of the next one, by chunk parity
-        bool sp[2] = {false, false};
-        unsigned vl[2] = {0u, 0u};
-        constexpr unsigned ALL = (1u << EPC) - 1u;
-        StagePlan pl;  // where the chunk fetched by the current iteration comes from
-        __syncthreads();  // the list in LDS is complete
-        chunk_entries(0, col, valid, part);
-        stage_chunk(0, col);
-        sp[0] = part != 0u || valid != ALL;
-        vl[0] = valid;
-        if (sp[0]) load_mask(col, mk[0]);
-        chunk_entries(1 < T ? 1 : 0, coln, valid, part);
-        sp[1] = 1 < T && (part != 0u || valid != ALL);
-        vl[1] = valid;
-        plan_chunk(coln, pl);
-        int raw[EPC];  // list entries of the chunk after next, read ahead
-        entries_read(2 < T ? 2 : T - 1, raw);
-#pragma unroll
-        for (int c = 0; c < D / 16; c++) asm volatile("" ::"v"(qf[c]));
-        if (sp[0]) settle(mk[0]);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        // Two chunks per trip so that the LDS stage is a compile-time constant.  Iteration tc computes chunk tc
-        // while chunk tc+1 is fetched (its pieces go out between the S bundles) and, during the P.V phase, turns
-        // the list entries of chunk tc+2 into the fetch plan of the next iteration.  Indices past the last chunk
-        // are clamped to it: the values are computed and never used.
-        for (int t = 0; t < T; t += 2) {
-            static_for<2>([&](auto jc) {
-                constexpr int j = decltype(jc)::value;
-                constexpr int cur = j & 1, nxt = cur ^ 1;
-                const int tc = t + j;
-                if (tc < T) {
-                    const bool fetch = tc + 1 < T;
-                    if (sp[nxt]) load_mask(coln, mk[nxt]);
-                    f32x16 s[2];
-                    phase_s(jc, s, std::integral_constant<int, nxt>{}, fetch, pl);
-                    const int t2 = tc + 2 < T ? tc + 2 : T - 1, t3 = tc + 3 < T ? tc + 3 : T - 1;
-                    int col2[EPC];
-                    unsigned valid2 = 0u, part2 = 0u;
-                    StagePlan pl2;
-                    phase_pv(jc, s, sp[cur], vl[cur], mk[cur], [&](int b, int nb) {
-                        const int per = (2 * EPC + nb - 1) / nb;  // plan entries per bundle
-                        if (b == 0) entries_use(t2, raw, col2, valid2, part2);
-#pragma unroll
-                        for (int i = b * per; i < (b + 1) * per && i < 2 * EPC; i++) {
-                            if (i & 1) pl2.vp[i >> 1] = vbase + (int64_t)col2[i >> 1] * p.vs[2];
-                            else pl2.kp[i >> 1] = kbase + (int64_t)col2[i >> 1] * p.ks[2];
-                        }
-                        if (b == nb - 1) entries_read(t3, raw);
-                    });
-                    pl = pl2;
-#pragma unroll
-                    for (int e = 0; e < EPC; e++) coln[e] = col2[e];
-                    // chunk tc+2 will be computed from the slot of chunk tc
-                    const bool sp2 = tc + 2 < T && (part2 != 0u || valid2 != ALL);
-                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // chunk tc+1 and its mask words have landed
-                    if (sp[nxt]) settle(mk[nxt]);
-                    sp[cur] = sp2;
-                    vl[cur] = valid2;
-                    __syncthreads();
-                }
-            });
-        }
-    }
-
-    // Epilogue: O = acc / l (sparse_attn_kernel.py:144); rows that attended to nothing give 0.
-    const float l_tot = l32 < 16 ? acc_l[0] : acc_l[1];
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    uint16_t *orow = p.o + b * p.os[0] + h * p.os[1] + (int64_t)qrow * p.os[2] + 4 * hh;
-#pragma unroll
-    for (int db = 0; db < D / 32; db++)
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const u32x2 w = {E::pack2(acc[db][4 * g] * inv, acc[db][4 * g + 1] * inv),
-                             E::pack2(acc[db][4 * g + 2] * inv, acc[db][4 * g + 3] * inv)};
-            *(u32x2 *)(orow + 32 * db + 8 * g) = w;
-        }
-}
-
-template <int DT, int D, int NW, int MODE>
-hipError_t launch_one(const FwdParams &p, hipStream_t stream) {
-    // Eight waves fill a CU's register file on their own, so that workgroup can have most of the LDS: 4 stages.
-    constexpr int NS = NW == 8 ? 4 : 2;
-    constexpr int smem = 2 * NS * 64 * D * 2 + kListCap * 4;  // NS stages of 64 rows for K and for V + the list
-    auto kern = sparse_fwd_kernel<DT, D, NW, MODE, NS, NW == 8>;
-    static bool attr_set = false;  // benign race: every thread sets the same value
-    if (!attr_set) {
-        const hipError_t e =
-            hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
-    const unsigned grid = (unsigned)p.nQ * (unsigned)p.B * (unsigned)p.H;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), smem, stream, p);
-    return hipGetLastError();
-}
-
-template <int DT, int D, int NW>
-hipError_t launch_mode(const FwdParams &p, hipStream_t stream) {
-    if (p.BK == 16) return launch_one<DT, D, NW, 0>(p, stream);
-    if (p.BK == 32) return launch_one<DT, D, NW, 1>(p, stream);
-    return launch_one<DT, D, NW, 2>(p, stream);
-}
-
-template <int DT, int D>
-hipError_t launch_bq(const FwdParams &p, int BQ, hipStream_t stream) {
-    switch (BQ) {
-        case 32: return launch_mode<DT, D, 1>(p, stream);
-        case 64: return launch_mode<DT, D, 2>(p, stream);
-        case 128: return launch_mode<DT, D, 4>(p, stream);
-        case 256: return launch_mode<DT, D, 8>(p, stream);
-        default: return hipErrorInvalidValue;
-    }
-}
-
-template <int DT>
-hipError_t launch_d(const FwdParams &p, int D, int BQ, hipStream_t stream) {
-    switch (D) {
-        case 64: return launch_bq<DT, 64>(p, BQ, stream);
-        case 128: return launch_bq<DT, 128>(p, BQ, stream);
-        default: return hipErrorInvalidValue;
-    }
-}
-
-}  // namespace
+template <int DT, bool PK>
+hipError_t launch_fwd_variant(const FwdParams &p, int D, int BQ, hipStream_t stream);
+extern template hipError_t launch_fwd_variant<0, false>(const FwdParams &, int, int, hipStream_t);
+extern template hipError_t launch_fwd_variant<0, true>(const FwdParams &, int, int, hipStream_t);
+extern template hipError_t launch_fwd_variant<1, false>(const FwdParams &, int, int, hipStream_t);
+extern template hipError_t launch_fwd_variant<1, true>(const FwdParams &, int, int, hipStream_t);
 
 hipError_t launch_fwd(const FwdParams &p, int dtype, int D, int BQ, hipStream_t stream) {
-    if (dtype == 0) return launch_d<0>(p, D, BQ, stream);
-    if (dtype == 1) return launch_d<1>(p, D, BQ, stream);
+    const bool pk = p.packed != nullptr;
+    if (dtype == 0) return pk ? launch_fwd_variant<0, true>(p, D, BQ, stream) : launch_fwd_variant<0, false>(p, D, BQ, stream);
+    if (dtype == 1) return pk ? launch_fwd_variant<1, true>(p, D, BQ, stream) : launch_fwd_variant<1, false>(p, D, BQ, stream);
     return hipErrorInvalidValue;
 }
 

@@ -134,19 +134,25 @@ int sa_mask_classify(const uint8_t *mask, const int64_t mask_strides[4], int B, 
     return SA_OK;
 }
 
-int sa_sparse_attention_fwd(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
-                            const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
-                            const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
-                            const int64_t full_ids_strides[4], const int32_t *full_lens,
-                            const int64_t full_lens_strides[3], const int32_t *part_ids,
-                            const int64_t part_ids_strides[4], const int32_t *part_lens,
-                            const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int D, int BQ, int BK,
-                            int dtype, float sm_scale_log2, void *stream) {
+}  // extern "C"
+
+namespace {
+
+int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4], const void *v,
+                 const int64_t v_strides[4], void *o, const int64_t o_strides[4], const uint8_t *mask,
+                 const int64_t mask_strides[4], const int32_t *full_ids, const int64_t full_ids_strides[4],
+                 const int32_t *full_lens, const int64_t full_lens_strides[3], const int32_t *part_ids,
+                 const int64_t part_ids_strides[4], const int32_t *part_lens, const int64_t part_lens_strides[3],
+                 const uint8_t *packed, const int64_t packed_strides[2], bool use_packed, int B, int H, int Sq, int Sk,
+                 int D, int BQ, int BK, int dtype, float sm_scale_log2, void *stream) {
     g_error[0] = 0;
-    if (!q || !k || !v || !o || !mask || !q_strides || !k_strides || !v_strides || !o_strides || !mask_strides ||
-        !full_ids || !full_ids_strides || !full_lens || !full_lens_strides || !part_ids || !part_ids_strides ||
-        !part_lens || !part_lens_strides)
+    if (!q || !k || !v || !o || !q_strides || !k_strides || !v_strides || !o_strides || !full_ids ||
+        !full_ids_strides || !full_lens || !full_lens_strides || !part_ids || !part_ids_strides || !part_lens ||
+        !part_lens_strides)
         return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd: null pointer argument");
+    if (use_packed ? (!packed || !packed_strides) : (!mask || !mask_strides))
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd: null pointer argument (%s)",
+                    use_packed ? "packed" : "mask");
     if (const int rc = check_tiling(B, H, Sq, Sk, BQ, BK)) return rc;
     if (D <= 0) return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd: D must be positive (got %d)", D);
     if (!(sm_scale_log2 > 0.f) || !(sm_scale_log2 < 3.0e38f))
@@ -191,10 +197,14 @@ int sa_sparse_attention_fwd(const void *q, const int64_t q_strides[4], const voi
         fp.pls[i] = part_lens_strides[i];
     }
     for (int i = 0; i < 4; i++) {
-        fp.ms[i] = mask_strides[i];
+        fp.ms[i] = mask_strides ? mask_strides[i] : 0;
         fp.fis[i] = full_ids_strides[i];
         fp.pis[i] = part_ids_strides[i];
     }
+    fp.packed = use_packed ? packed : nullptr;
+    fp.pks[0] = use_packed ? packed_strides[0] : 0;
+    fp.pks[1] = use_packed ? packed_strides[1] : 0;
+    fp.nK = Sk / BK;
     fp.B = B;
     fp.H = H;
     fp.Sq = Sq;
@@ -202,13 +212,119 @@ int sa_sparse_attention_fwd(const void *q, const int64_t q_strides[4], const voi
     fp.nQ = Sq / BQ;
     fp.BK = BK;
     fp.lbk = lbk;
-    fp.mask_vec4 = (mask_strides[3] == 1 && aligned(mask, 4) && mask_strides[0] % 4 == 0 && mask_strides[1] % 4 == 0 &&
-                    mask_strides[2] % 4 == 0)
+    fp.mask_vec4 = (!use_packed && mask_strides[3] == 1 && aligned(mask, 4) && mask_strides[0] % 4 == 0 &&
+                    mask_strides[1] % 4 == 0 && mask_strides[2] % 4 == 0)
                        ? 1
                        : 0;
     fp.scale = sm_scale_log2;
     const hipError_t e = sa::launch_fwd(fp, dtype, D, BQ, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_fwd: launch failed: %s", hipGetErrorString(e));
+    return SA_OK;
+}
+
+// Distinct planes of a mask along b and h, and whether `strides` may fold them.
+struct Planes {
+    int uB, uH;
+    bool bcast_b, bcast_h;
+};
+Planes planes_of(const int64_t mask_strides[4], int B, int H) {
+    Planes pl;
+    pl.bcast_b = mask_strides[0] == 0 || B == 1;
+    pl.bcast_h = mask_strides[1] == 0 || H == 1;
+    pl.uB = pl.bcast_b ? 1 : B;
+    pl.uH = pl.bcast_h ? 1 : H;
+    return pl;
+}
+
+}  // namespace
+
+extern "C" {
+
+int sa_sparse_attention_fwd(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                            const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
+                            const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
+                            const int64_t full_ids_strides[4], const int32_t *full_lens,
+                            const int64_t full_lens_strides[3], const int32_t *part_ids,
+                            const int64_t part_ids_strides[4], const int32_t *part_lens,
+                            const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int D, int BQ, int BK,
+                            int dtype, float sm_scale_log2, void *stream) {
+    return forward_impl(q, q_strides, k, k_strides, v, v_strides, o, o_strides, mask, mask_strides, full_ids,
+                        full_ids_strides, full_lens, full_lens_strides, part_ids, part_ids_strides, part_lens,
+                        part_lens_strides, nullptr, nullptr, false, B, H, Sq, Sk, D, BQ, BK, dtype, sm_scale_log2,
+                        stream);
+}
+
+int sa_sparse_attention_fwd_packed(const void *q, const int64_t q_strides[4], const void *k,
+                                   const int64_t k_strides[4], const void *v, const int64_t v_strides[4], void *o,
+                                   const int64_t o_strides[4], const uint8_t *mask, const int64_t mask_strides[4],
+                                   const int32_t *full_ids, const int64_t full_ids_strides[4],
+                                   const int32_t *full_lens, const int64_t full_lens_strides[3],
+                                   const int32_t *part_ids, const int64_t part_ids_strides[4],
+                                   const int32_t *part_lens, const int64_t part_lens_strides[3],
+                                   const uint8_t *packed, const int64_t packed_strides[2], int B, int H, int Sq,
+                                   int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2, void *stream) {
+    if (packed && packed_strides) {
+        if ((B > 1 && packed_strides[0] % 4) || (H > 1 && packed_strides[1] % 4) || !aligned(packed, 4)) {
+            g_error[0] = 0;
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd_packed: packed needs a 4-byte aligned base and plane strides");
+        }
+    }
+    return forward_impl(q, q_strides, k, k_strides, v, v_strides, o, o_strides, mask, mask_strides, full_ids,
+                        full_ids_strides, full_lens, full_lens_strides, part_ids, part_ids_strides, part_lens,
+                        part_lens_strides, packed, packed_strides, true, B, H, Sq, Sk, D, BQ, BK, dtype,
+                        sm_scale_log2, stream);
+}
+
+size_t sa_mask_pack_partial_bytes(const int64_t mask_strides[4], int B, int H, int Sq, int Sk, int BQ, int BK) {
+    if (!mask_strides || check_tiling(B, H, Sq, Sk, BQ, BK) != SA_OK || BK % 8) return 0;
+    const Planes pl = planes_of(mask_strides, B, H);
+    return (size_t)pl.uB * pl.uH * (size_t)Sq * (size_t)Sk / 8;
+}
+
+int sa_mask_pack_partial(const uint8_t *mask, const int64_t mask_strides[4], int B, int H, int Sq, int Sk, int BQ,
+                         int BK, const int32_t *part_ids, const int64_t part_ids_strides[4],
+                         const int32_t *part_lens, const int64_t part_lens_strides[3], uint8_t *packed,
+                         const int64_t packed_strides[2], void *stream) {
+    g_error[0] = 0;
+    if (!mask || !mask_strides || !part_ids || !part_ids_strides || !part_lens || !part_lens_strides || !packed ||
+        !packed_strides)
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_pack_partial: null pointer argument");
+    if (const int rc = check_tiling(B, H, Sq, Sk, BQ, BK)) return rc;
+    if (BK % 8) return fail(SA_ERR_UNSUPPORTED, "sa_mask_pack_partial: BLOCK_K %d (must be a multiple of 8)", BK);
+    const Planes pl = planes_of(mask_strides, B, H);
+    const int64_t plane_bytes = (int64_t)Sq * Sk / 8;
+    if ((pl.uB > 1 && packed_strides[0] < plane_bytes) || (pl.uH > 1 && packed_strides[1] < plane_bytes))
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_pack_partial: packed planes overlap (strides %lld, %lld; %lld bytes per plane)",
+                    (long long)packed_strides[0], (long long)packed_strides[1], (long long)plane_bytes);
+    const int nQ = Sq / BQ, nK = Sk / BK;
+    if (nQ > 65535 || (int64_t)pl.uB * pl.uH > 65535)
+        return fail(SA_ERR_UNSUPPORTED, "sa_mask_pack_partial: more than 65535 Q tiles or distinct mask planes");
+
+    sa::PackParams pp{};
+    pp.mask = mask;
+    pp.sb = mask_strides[0];
+    pp.sh = mask_strides[1];
+    pp.sq = mask_strides[2];
+    pp.sk = mask_strides[3];
+    pp.part_ids = part_ids;
+    pp.part_lens = part_lens;
+    for (int i = 0; i < 4; i++) pp.pis[i] = part_ids_strides[i];
+    for (int i = 0; i < 3; i++) pp.pls[i] = part_lens_strides[i];
+    pp.packed = packed;
+    pp.ob = packed_strides[0];
+    pp.oh = packed_strides[1];
+    pp.uB = pl.uB;
+    pp.uH = pl.uH;
+    pp.BQ = BQ;
+    pp.BK = BK;
+    pp.nQ = nQ;
+    pp.nK = nK;
+    pp.vec8 = ((pp.sk == 1 || Sk == 1) && aligned(mask, 8) && pp.sq % 8 == 0 && (pl.uB == 1 || pp.sb % 8 == 0) &&
+               (pl.uH == 1 || pp.sh % 8 == 0))
+                  ? 1
+                  : 0;
+    const hipError_t e = sa::launch_pack(pp, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_mask_pack_partial: launch failed: %s", hipGetErrorString(e));
     return SA_OK;
 }
 

@@ -6,6 +6,7 @@ Mirrors the interface of the reference's ``sparseattention/mask_utils.py``:
 from __future__ import annotations
 
 from dataclasses import dataclass
+from typing import Optional
 
 import torch
 
@@ -20,12 +21,19 @@ class MaskMetadata:
     ``unmasked_lens``  int32 [B,H,Sq/BQ]: how many leading slots of it are valid;
     ``masked_kv_ids`` / ``masked_lens``: the same for tiles with some but not all entries True.
     Slots past the count hold unspecified values.
+
+    ``packed_masks`` is an addition to the reference's four fields (optional, last, default None, so code
+    that builds the dataclass positionally keeps working): uint8 [B,H,Sq/BQ,Sk/BK,BQ*BK/8], the mask entries of
+    the PARTIAL tiles at one bit each.  ``packed_masks[b,h,qt,slot]`` belongs to KV tile
+    ``masked_kv_ids[b,h,qt,slot]``: rows first, entry (r, c) in bit ``c & 7`` of byte ``(r*BK + c) >> 3``.
+    When present, :func:`sparse_attention` reads these bits and never touches the bool mask.
     """
 
     unmasked_kv_ids: torch.Tensor
     unmasked_lens: torch.Tensor
     masked_kv_ids: torch.Tensor
     masked_lens: torch.Tensor
+    packed_masks: Optional[torch.Tensor] = None
 
 
 def _check_mask(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int):
@@ -67,13 +75,17 @@ def compute_mask_slow(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int) -> MaskMet
     return MaskMetadata(fid, fl, pid, pl)
 
 
-def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int) -> MaskMetadata:
+def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int,
+                        pack_partial: Optional[bool] = None) -> MaskMetadata:
     """Classify the mask's tiles on the GPU (replaces mask_utils.py:85-107).
 
     ``mask``: bool [B,H,Sq,Sk] on a ROCm device, any strides.  Dimensions that are broadcast in
     ``mask`` (stride 0, e.g. from ``mask.expand(B,H,Sq,Sk)``) are classified once and the returned
     tensors are broadcast views over them, so every ``[b,h]`` plane reads the same values the
     reference would have written there.
+
+    ``pack_partial``: also fill ``MaskMetadata.packed_masks`` (Sq*Sk/8 bytes per distinct mask plane).
+    Default: whenever BLOCK_K is a multiple of 8; ``False`` gives exactly the reference's four tensors.
     """
     B, H, Sq, Sk = _check_mask(mask, BLOCK_Q, BLOCK_K)
     if not mask.is_cuda:
@@ -103,7 +115,22 @@ def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int) -> MaskM
         # the kernels run on the current stream; the caching allocator may hand this block out again
         # only to work queued after them on the same stream, so dropping the reference here is safe
         del workspace
-    return MaskMetadata(fid, fl, pid, pl)
+        packed = None
+        if pack_partial is None:
+            pack_partial = BLOCK_K % 8 == 0
+        if pack_partial:
+            if BLOCK_K % 8:
+                raise ValueError(f"pack_partial needs BLOCK_K to be a multiple of 8 (got {BLOCK_K})")
+            packed = torch.empty(uB, uH, nQ, nK, BLOCK_Q * BLOCK_K // 8, dtype=torch.uint8, device=dev)
+            rc = lib.sa_mask_pack_partial(
+                mask.data_ptr(), ms, B, H, Sq, Sk, BLOCK_Q, BLOCK_K,
+                pid.data_ptr(), _native.strides(pid.stride()), pl.data_ptr(), _native.strides(pl.stride()),
+                packed.data_ptr(), _native.strides(packed.stride()[:2]),
+                torch.cuda.current_stream(dev).cuda_stream,
+            )
+            _native.check(rc)
+            packed = packed.expand(B, H, nQ, nK, BLOCK_Q * BLOCK_K // 8)
+    return MaskMetadata(fid, fl, pid, pl, packed)
 
 
 # Tile sizes tried by select_block_sizes, and what one executed mask entry costs at each BLOCK_Q relative to

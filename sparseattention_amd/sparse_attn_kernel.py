@@ -53,19 +53,28 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
     assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
     if mask.device != q.device:
         raise ValueError("mask must be on the same device as q")
+    packed = getattr(mask_metadata, "packed_masks", None)
+    if packed is not None:
+        shape = (B, H, nQ, nK, BLOCK_Q * BLOCK_K // 8)
+        if (tuple(packed.shape) != shape or packed.dtype != torch.uint8 or packed.device != q.device
+                or packed.stride()[2:] != (nK * shape[4], shape[4], 1)):
+            raise ValueError(f"mask_metadata.packed_masks: expected uint8 {shape} on {q.device} with contiguous "
+                             f"tiles, got {packed.dtype} {tuple(packed.shape)} strides {packed.stride()}")
 
     qc, kc, vc = _kernel_ready(q), _kernel_ready(k), _kernel_ready(v)
     o = torch.empty_like(qc)
     lib = _native.load()
     S = _native.strides
     with torch.cuda.device(q.device):
-        rc = lib.sa_sparse_attention_fwd(
-            qc.data_ptr(), S(qc.stride()), kc.data_ptr(), S(kc.stride()), vc.data_ptr(), S(vc.stride()),
-            o.data_ptr(), S(o.stride()), mask.data_ptr(), S(mask.stride()),
-            fid.data_ptr(), S(fid.stride()), fl.data_ptr(), S(fl.stride()),
-            pid.data_ptr(), S(pid.stride()), pl.data_ptr(), S(pl.stride()),
-            B, H, Sq, Sk, D, int(BLOCK_Q), int(BLOCK_K), _DTYPES[q.dtype], sm_scale,
-            torch.cuda.current_stream(q.device).cuda_stream,
-        )
+        common = (qc.data_ptr(), S(qc.stride()), kc.data_ptr(), S(kc.stride()), vc.data_ptr(), S(vc.stride()),
+                  o.data_ptr(), S(o.stride()), mask.data_ptr(), S(mask.stride()),
+                  fid.data_ptr(), S(fid.stride()), fl.data_ptr(), S(fl.stride()),
+                  pid.data_ptr(), S(pid.stride()), pl.data_ptr(), S(pl.stride()))
+        tail = (B, H, Sq, Sk, D, int(BLOCK_Q), int(BLOCK_K), _DTYPES[q.dtype], sm_scale,
+                torch.cuda.current_stream(q.device).cuda_stream)
+        if packed is not None:
+            rc = lib.sa_sparse_attention_fwd_packed(*common, packed.data_ptr(), S(packed.stride()[:2]), *tail)
+        else:
+            rc = lib.sa_sparse_attention_fwd(*common, *tail)
     _native.check(rc)
     return o

@@ -99,6 +99,48 @@ def test_forward_rejects_bad_arguments():
     assert fwd(qs=_native.strides((256 * 128, 256 * 128, 132, 1))) == _native.SA_ERR_UNSUPPORTED
 
 
+def pack(mask=FAKE, ms=S4, B=1, H=1, Sq=64, Sk=64, BQ=32, BK=32, ids=FAKE, packed=FAKE, ps=None):
+    lib = _native.load()
+    ps = ps or _native.strides((0, 0))
+    return lib.sa_mask_pack_partial(mask, ms, B, H, Sq, Sk, BQ, BK, ids, I4, FAKE, S3, packed, ps, None)
+
+
+def test_pack_rejects_bad_arguments_and_sizes_its_buffer():
+    lib = _native.load()
+    f = lib.sa_mask_pack_partial_bytes
+    assert f(_native.strides((0, 0, 4096, 1)), 8, 32, 4096, 4096, 128, 32) == 4096 * 4096 // 8
+    assert f(_native.strides((1 << 24, 0, 4096, 1)), 8, 32, 4096, 4096, 128, 32) == 8 * 4096 * 4096 // 8
+    assert f(_native.strides((0, 0, 4096, 1)), 8, 32, 4096, 4096, 128, 4) == 0      # BLOCK_K % 8
+    assert f(_native.strides((0, 0, 4096, 1)), 8, 32, 4096, 4096, 100, 32) == 0
+    assert pack(mask=None) == _native.SA_ERR_INVALID_ARGUMENT and "null" in last_error()
+    assert pack(packed=None) == _native.SA_ERR_INVALID_ARGUMENT
+    assert pack(ids=None) == _native.SA_ERR_INVALID_ARGUMENT
+    assert pack(Sq=65) == _native.SA_ERR_INVALID_ARGUMENT and "BLOCK_Q" in last_error()
+    assert pack(BK=4) == _native.SA_ERR_UNSUPPORTED and "multiple of 8" in last_error()
+    # two distinct batch planes need room for two packed planes
+    assert pack(B=2, ms=_native.strides((4096, 0, 64, 1)), ps=_native.strides((8, 0))) == _native.SA_ERR_INVALID_ARGUMENT
+    assert "overlap" in last_error()
+
+
+def test_packed_forward_rejects_bad_arguments():
+    lib = _native.load()
+    qs = _native.strides((256 * 128, 256 * 128, 128, 1))
+
+    def call(packed=FAKE, ps=_native.strides((0, 0)), mask=None, BK=32, B=1):
+        return lib.sa_sparse_attention_fwd_packed(FAKE, qs, FAKE, qs, FAKE, qs, FAKE, qs, mask, None, FAKE, I4, FAKE,
+                                                  S3, FAKE, I4, FAKE, S3, packed, ps, B, 1, 256, 256, 128, 128, BK, 0,
+                                                  0.1, None)
+
+    assert call(packed=None) == _native.SA_ERR_INVALID_ARGUMENT and "packed" in last_error()
+    assert call(ps=None) == _native.SA_ERR_INVALID_ARGUMENT
+    assert call(packed=FAKE + 2) == _native.SA_ERR_UNSUPPORTED and "aligned" in last_error()
+    assert call(B=2, ps=_native.strides((6, 0))) == _native.SA_ERR_UNSUPPORTED
+    assert call(BK=8) == _native.SA_ERR_UNSUPPORTED and "BLOCK_K" in last_error()
+    # the plain entry point still insists on a mask
+    assert lib.sa_sparse_attention_fwd(FAKE, qs, FAKE, qs, FAKE, qs, FAKE, qs, None, None, FAKE, I4, FAKE, S3, FAKE, I4,
+                                       FAKE, S3, 1, 1, 256, 256, 128, 128, 32, 0, 0.1, None) == _native.SA_ERR_INVALID_ARGUMENT
+
+
 def test_python_wrappers_refuse_to_run_without_a_gpu_tensor():
     from sparseattention_amd import compute_mask_kernel, sparse_attention
 
