@@ -8,10 +8,12 @@
  *                             (sparseattention/mask_utils.py:85-107, kernel :47-82)
  *   sa_sparse_attention_fwd   replaces the launch in sparse_attention
  *                             (sparseattention/sparse_attn_kernel.py:149-185, kernels :10-63, :74-146)
- *   sa_mask_pack_partial, sa_sparse_attention_fwd_packed
- *                             an optional faster route for the PARTIAL tiles: their mask entries are
- *                             packed to one bit each once per mask, and the forward reads those bits
- *                             instead of the mask tile loads of sparse_attn_kernel.py:42-46
+ *   sa_mask_pack_partial, sa_fwd_schedule, sa_sparse_attention_fwd_ex
+ *                             optional accelerators of the same forward, prepared once per mask: the mask
+ *                             entries of PARTIAL tiles packed to one bit each (read instead of the mask tile
+ *                             loads of sparse_attn_kernel.py:42-46), and a schedule that deals the Q tiles
+ *                             out to workgroups that stay resident (instead of the grid of
+ *                             sparse_attn_kernel.py:167)
  *
  * Conventions
  *   - All pointers are DEVICE pointers owned by the caller.  The library allocates nothing,
@@ -36,7 +38,7 @@
 extern "C" {
 #endif
 
-#define SA_ABI_VERSION 2
+#define SA_ABI_VERSION 3
 
 enum sa_status {
     SA_OK = 0,
@@ -145,20 +147,44 @@ int sa_mask_pack_partial(const uint8_t *mask, const int64_t mask_strides[4], int
                          const int64_t packed_strides[2], void *stream);
 
 /*
- * sa_sparse_attention_fwd with the PARTIAL tiles' mask entries taken from `packed` (the output of
- * sa_mask_pack_partial for the same mask, tile sizes and lists; packed_strides may be 0 on broadcast
- * dimensions).  `mask` is not read and may be NULL, so the bool tensor can be released once the lists and
- * the packed bits exist.  Results are bit-identical to sa_sparse_attention_fwd.
+ * Schedule of the forward's persistent workgroups.  No counterpart in the reference, whose grid is one program
+ * per Q tile (sparse_attn_kernel.py:167): here a grid that fills the device once walks over the Q tiles, so that
+ * the start-up latencies of a workgroup (arguments, counts, lists, first K/V tiles) are not paid per Q tile, and
+ * the tiles are dealt out by their known cost (the list lengths) instead of in launch order.
+ *
+ * sa_fwd_schedule_bytes   size of the schedule buffer for this problem on the CURRENT device (it depends on the
+ *                         number of compute units); 0 when the forward has no persistent kernel for the tile
+ *                         sizes (BQ must be 32, 64 or 128, BK a power of two >= 16 with Sk/BK <= 1024) or on
+ *                         invalid arguments.
+ * sa_fwd_schedule         fills it from the two count tensors of sa_mask_classify (same stream, after it).  The
+ *                         result depends on the counts, B, H, the tile sizes and the device only: compute it
+ *                         once per mask and reuse it for every forward over that mask.
  */
-int sa_sparse_attention_fwd_packed(const void *q, const int64_t q_strides[4], const void *k,
-                                   const int64_t k_strides[4], const void *v, const int64_t v_strides[4], void *o,
-                                   const int64_t o_strides[4], const uint8_t *mask, const int64_t mask_strides[4],
-                                   const int32_t *full_ids, const int64_t full_ids_strides[4],
-                                   const int32_t *full_lens, const int64_t full_lens_strides[3],
-                                   const int32_t *part_ids, const int64_t part_ids_strides[4],
-                                   const int32_t *part_lens, const int64_t part_lens_strides[3],
-                                   const uint8_t *packed, const int64_t packed_strides[2], int B, int H, int Sq,
-                                   int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2, void *stream);
+size_t sa_fwd_schedule_bytes(int B, int H, int Sq, int Sk, int BQ, int BK);
+int sa_fwd_schedule(const int32_t *full_lens, const int64_t full_lens_strides[3], const int32_t *part_lens,
+                    const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int BQ, int BK,
+                    int32_t *schedule, size_t schedule_bytes, void *stream);
+
+/*
+ * sa_sparse_attention_fwd with the optional accelerators; results are bit-identical to it.
+ *
+ *   packed, packed_strides   output of sa_mask_pack_partial for the same mask, tile sizes and lists (strides may
+ *                            be 0 on broadcast dimensions), or NULL.  When given, `mask` is not read and may be
+ *                            NULL, so the bool tensor can be released once the lists and the packed bits exist.
+ *   schedule, schedule_bytes output of sa_fwd_schedule for the same counts and sizes on this device, or NULL
+ *                            (then, and when schedule_bytes is not sa_fwd_schedule_bytes(...), one workgroup
+ *                            per Q tile is launched as in sa_sparse_attention_fwd).
+ */
+int sa_sparse_attention_fwd_ex(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                               const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
+                               const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
+                               const int64_t full_ids_strides[4], const int32_t *full_lens,
+                               const int64_t full_lens_strides[3], const int32_t *part_ids,
+                               const int64_t part_ids_strides[4], const int32_t *part_lens,
+                               const int64_t part_lens_strides[3], const uint8_t *packed,
+                               const int64_t packed_strides[2], const int32_t *schedule, size_t schedule_bytes, int B,
+                               int H, int Sq, int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2,
+                               void *stream);
 
 #ifdef __cplusplus
 }

@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsparseattn_hip.so")
 
-SA_ABI_VERSION = 2
+SA_ABI_VERSION = 3
 SA_OK = 0
 SA_ERR_INVALID_ARGUMENT = -1
 SA_ERR_UNSUPPORTED = -2
@@ -29,7 +29,9 @@ EXPORTS = (
     "sa_sparse_attention_fwd",
     "sa_mask_pack_partial_bytes",
     "sa_mask_pack_partial",
-    "sa_sparse_attention_fwd_packed",
+    "sa_fwd_schedule_bytes",
+    "sa_fwd_schedule",
+    "sa_sparse_attention_fwd_ex",
 )
 
 _lib = None
@@ -75,9 +77,14 @@ def load() -> ctypes.CDLL:
     lib.sa_mask_pack_partial_bytes.argtypes = [_i64p] + [ctypes.c_int] * 6
     lib.sa_mask_pack_partial.restype = ctypes.c_int
     lib.sa_mask_pack_partial.argtypes = [_vp, _i64p] + [ctypes.c_int] * 6 + [_vp, _i64p] * 3 + [_vp]
-    lib.sa_sparse_attention_fwd_packed.restype = ctypes.c_int
-    lib.sa_sparse_attention_fwd_packed.argtypes = (
-        [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [_vp, _i64p] + [ctypes.c_int] * 8 + [ctypes.c_float, _vp]
+    lib.sa_fwd_schedule_bytes.restype = ctypes.c_size_t
+    lib.sa_fwd_schedule_bytes.argtypes = [ctypes.c_int] * 6
+    lib.sa_fwd_schedule.restype = ctypes.c_int
+    lib.sa_fwd_schedule.argtypes = [_vp, _i64p] * 2 + [ctypes.c_int] * 6 + [_vp, ctypes.c_size_t, _vp]
+    lib.sa_sparse_attention_fwd_ex.restype = ctypes.c_int
+    lib.sa_sparse_attention_fwd_ex.argtypes = (
+        [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, ctypes.c_size_t]
+        + [ctypes.c_int] * 8 + [ctypes.c_float, _vp]
     )
     if lib.sa_abi_version() != SA_ABI_VERSION:
         raise RuntimeError(f"libsparseattn_hip ABI {lib.sa_abi_version()} != expected {SA_ABI_VERSION}")

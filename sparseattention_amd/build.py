@@ -20,9 +20,10 @@ LIB_PATH = os.path.join(_HERE, "libsparseattn_hip.so")
 # (source, object name, extra defines).  The forward kernels are one source compiled per element type and
 # mask source, so that the variants build in parallel.
 UNITS = [("sparseattn_api.hip", "sparseattn_api.o", []), ("mask_classify.hip", "mask_classify.o", []),
-         ("sparse_fwd.hip", "sparse_fwd.o", [])]
-UNITS += [("sparse_fwd_inst.hip", f"sparse_fwd_dt{dt}_pk{pk}.o", [f"-DSA_FWD_DT={dt}", f"-DSA_FWD_PK={pk}"])
-          for dt in (0, 1) for pk in (0, 1)]
+         ("fwd_schedule.hip", "fwd_schedule.o", []), ("sparse_fwd.hip", "sparse_fwd.o", [])]
+UNITS += [("sparse_fwd_inst.hip", f"sparse_fwd_dt{dt}_pk{pk}_ps{ps}.o",
+           [f"-DSA_FWD_DT={dt}", f"-DSA_FWD_PK={pk}", f"-DSA_FWD_PS={ps}"])
+          for dt in (0, 1) for pk in (0, 1) for ps in (0, 1)]
 
 # -packed-fp32-ops is switched off on purpose: the compiler must not form v_pk_*_f32 from float code.
 HIPCC_FLAGS = [

@@ -132,6 +132,8 @@ constexpr float kMaxSlack = 8.0f;
 
 // List entries kept in LDS per Q tile (8 KiB); longer lists are read from global memory per chunk.
 constexpr int kListCap = 2048;
+// Persistent workgroups keep two lists in the same space, of the Q tile at hand and of the next one.
+constexpr int kPsListCap = 1024;
 
 }  // namespace
 }  // namespace sa

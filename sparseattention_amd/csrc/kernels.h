@@ -40,7 +40,21 @@ struct PackParams {
     int vec8;  // 1: key stride 1 and every row segment 8-byte aligned, so 8 entries load as one qword
 };
 
+// Q tiles dealt out to G persistent workgroups (G a multiple of 8, G/8 <= 64).  Workgroup g = 8*j + x is taken
+// to run on XCD x (hardware hands consecutive workgroup ids to the XCDs in turn) and gets Q tiles of the x-th
+// eighth of the (b,h)-major order, so that the tiles sharing a K/V plane meet in one L2.
+// sched: int32 [G][R+1][4]; entry 0 of a row = {count, 0, 0, 0}, entries 1..count = {(b << 16) | h, qt, F, P}.
+struct ScheduleParams {
+    const int32_t *full_lens, *part_lens;
+    int64_t fls[3], pls[3];
+    int B, H, nQ;
+    int G, R;
+    int lbk;  // log2(BK): chunks of 64 keys per entry = BK/64, entries per chunk = 64/BK
+    int32_t *sched;
+};
+
 hipError_t launch_classify(const ClassifyParams &p, bool wide, hipStream_t stream);
+hipError_t launch_schedule(const ScheduleParams &p, hipStream_t stream);
 hipError_t launch_compact(const CompactParams &p, hipStream_t stream);
 hipError_t launch_pack(const PackParams &p, hipStream_t stream);
 
@@ -60,6 +74,9 @@ struct FwdParams {
     const uint8_t *packed;
     int64_t pks[2];  // bytes between packed planes along b and h (0 where the mask is broadcast)
     int nK;          // KV tiles per row of tiles (slots per Q tile in `packed`)
+    // Schedule of persistent workgroups (ScheduleParams layout), or null: then one workgroup per Q tile.
+    const int32_t *sched;
+    int sched_G, sched_R;  // workgroups, and entries per row after the header entry
     float scale;    // softmax scale / ln 2
 };
 

@@ -61,8 +61,14 @@ __device__ __forceinline__ void wait_vm_at_most(int n, int step) {
 // S phase while the other is in its P.V phase (see the main loop).
 // PK: the mask entries of PARTIAL tiles come bit-packed from p.packed (one bit per entry, rows first) instead of
 // from the bool mask.
-template <int DT, int D, int NW, int MODE, int NS, bool PP, bool PK>
+// PS: persistent workgroups.  The grid is as large as the device holds at once, and every workgroup walks its own
+// row of p.sched (Q tiles dealt out by schedule_kernel).  The chunk stream runs on across Q tiles: while the last
+// chunk of one tile is computed, the first chunk of the next is fetched and its queries are loaded, and the
+// lists of the tiles after that are on their way, so that the latencies a fresh workgroup would pay one after
+// the other (arguments, counts, lists, first K/V chunk) are paid once per workgroup instead of once per tile.
+template <int DT, int D, int NW, int MODE, int NS, bool PP, bool PK, bool PS>
 __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(const FwdParams p) {
+    static_assert(!PS || (!PP && NS == 2), "persistent workgroups use the two-stage loop");
     using E = Elem<DT>;
     constexpr int ROWB = D * 2;                   // bytes per K/V row in LDS
     constexpr int KBUF = 64 * ROWB, VBUF = 64 * ROWB;
@@ -86,44 +92,96 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
     // K/V plane run on the XCD whose L2 already holds it.  Planes are taken two at a time with their Q tiles
     // interleaved, last Q tile first (under causal-like masks it has the longest list): the slots that finish
     // the short tiles of one pair then pick up the long tiles of the next, which evens out the load.
-    const int total = gridDim.x, per = total >> 3;
-    int lin = blockIdx.x;
-    if (lin < (per << 3)) lin = (lin & 7) * per + (lin >> 3);
-    const int pair = lin / (2 * p.nQ), r = lin - pair * 2 * p.nQ;
-    const bool paired = 2 * pair + 1 < p.B * p.H;  // the last plane of an odd count goes alone
-    const int bh = 2 * pair + (paired ? (r & 1) : 0);
-    const int qt = p.nQ - 1 - (paired ? (r >> 1) : r);
-    const int b = bh / p.H, h = bh - b * p.H;
-
-    const uint16_t *kbase = p.k + b * p.ks[0] + h * p.ks[1];
-    const uint16_t *vbase = p.v + b * p.vs[0] + h * p.vs[1];
-    const int qrow = qt * (NW * 32) + wave * 32 + l32;  // the query row this lane owns
-    const uint8_t *mrow = p.mask + b * p.ms[0] + h * p.ms[1] + (int64_t)qrow * p.ms[2];
-    // this lane's row in the first packed tile of the Q tile: BK/8 bytes per row, NW*32 rows per tile
+    // The Q tile at hand: plane (b, h), tile qt, F FULL and NE - F PARTIAL entries, T chunks.  A persistent
+    // workgroup moves from tile to tile; the others keep the values they start with.
+    int b, h, qt, F, NE, T;
+    const uint16_t *kbase, *vbase;
+    const uint8_t *mrow, *prow;
+    const int32_t *fid, *pid;
+    int64_t orow_off;  // this lane's first output element
+    // this lane's row in a packed tile: BK/8 bytes per row, NW*32 rows per tile
     const int64_t tile_bytes = (int64_t)(NW * 4) * p.BK;
-    const uint8_t *prow = p.packed + b * p.pks[0] + h * p.pks[1] + (int64_t)qt * p.nK * tile_bytes +
-                          (wave * 32 + l32) * (p.BK >> 3);
     const int sh4 = 4 * hh;
-
-    const int32_t *fid = p.full_ids + b * p.fis[0] + h * p.fis[1] + qt * p.fis[2];
-    const int32_t *pid = p.part_ids + b * p.pis[0] + h * p.pis[1] + qt * p.pis[2];
-    const int F = p.full_lens[b * p.fls[0] + h * p.fls[1] + qt * p.fls[2]];
-    const int P = p.part_lens[b * p.pls[0] + h * p.pls[1] + qt * p.pls[2]];
-    const int NE = F + P;
-    const int T = MODE == 2 ? (NE << (p.lbk - 6)) : ((NE + EPC - 1) / EPC);
+    // what load_mask needs to know of a Q tile
+    struct MaskSrc {
+        const uint8_t *mrow, *prow;
+        int F, NE;
+    };
+    auto mask_src_of = [&](int b_, int h_, int qt_, int F_, int NE_) -> MaskSrc {
+        const int qrow_ = qt_ * (NW * 32) + wave * 32 + l32;  // the query row this lane owns
+        MaskSrc m;
+        m.mrow = p.mask + b_ * p.ms[0] + h_ * p.ms[1] + (int64_t)qrow_ * p.ms[2];
+        m.prow = p.packed + b_ * p.pks[0] + h_ * p.pks[1] + (int64_t)qt_ * p.nK * tile_bytes +
+                 (wave * 32 + l32) * (p.BK >> 3);
+        m.F = F_;
+        m.NE = NE_;
+        return m;
+    };
+    auto chunks_of = [&](int ne) -> int {
+        if constexpr (PS) {  // a tile without entries still runs one chunk of absent entries, which yields zeros
+            return MODE == 2 ? ((ne > 0 ? ne : 1) << (p.lbk - 6)) : (ne > 0 ? (ne + EPC - 1) / EPC : 1);
+        } else {
+            return MODE == 2 ? (ne << (p.lbk - 6)) : ((ne + EPC - 1) / EPC);
+        }
+    };
+    auto set_item = [&](int b_, int h_, int qt_, int F_, int P_) {
+        b = b_;
+        h = h_;
+        qt = qt_;
+        F = F_;
+        NE = F_ + P_;
+        T = chunks_of(NE);
+        kbase = p.k + b * p.ks[0] + h * p.ks[1];
+        vbase = p.v + b * p.vs[0] + h * p.vs[1];
+        const MaskSrc m = mask_src_of(b, h, qt, F, NE);
+        mrow = m.mrow;
+        prow = m.prow;
+        fid = p.full_ids + b * p.fis[0] + h * p.fis[1] + qt * p.fis[2];
+        pid = p.part_ids + b * p.pis[0] + h * p.pis[1] + qt * p.pis[2];
+        const int qrow_ = qt * (NW * 32) + wave * 32 + l32;
+        orow_off = b * p.os[0] + h * p.os[1] + (int64_t)qrow_ * p.os[2] + 4 * hh;
+    };
+    // Row of this workgroup in the schedule: entry 0 = {number of Q tiles, -, -, -}, then one entry
+    // {(b << 16) | h, qt, F, P} per Q tile.
+    const int4 *const sched_row = reinterpret_cast<const int4 *>(p.sched) + (int64_t)blockIdx.x * (p.sched_R + 1);
+    int n_items = 1;
+    if constexpr (PS) {
+        n_items = __builtin_amdgcn_readfirstlane(sched_row[0].x);
+        if (n_items <= 0) return;
+        const int4 e0 = sched_row[1];
+        const int bh0 = __builtin_amdgcn_readfirstlane(e0.x);
+        set_item(bh0 >> 16, bh0 & 0xffff, __builtin_amdgcn_readfirstlane(e0.y), __builtin_amdgcn_readfirstlane(e0.z),
+                 __builtin_amdgcn_readfirstlane(e0.w));
+    } else {
+        const int total = gridDim.x, per = total >> 3;
+        int lin = blockIdx.x;
+        if (lin < (per << 3)) lin = (lin & 7) * per + (lin >> 3);
+        const int pair = lin / (2 * p.nQ), r = lin - pair * 2 * p.nQ;
+        const bool paired = 2 * pair + 1 < p.B * p.H;  // the last plane of an odd count goes alone
+        const int bh = 2 * pair + (paired ? (r & 1) : 0);
+        const int qt0 = p.nQ - 1 - (paired ? (r >> 1) : r);
+        const int b0 = bh / p.H, h0 = bh - b0 * p.H;
+        set_item(b0, h0, qt0, p.full_lens[b0 * p.fls[0] + h0 * p.fls[1] + qt0 * p.fls[2]],
+                 p.part_lens[b0 * p.pls[0] + h0 * p.pls[1] + qt0 * p.pls[2]]);
+    }
 
     // Q^T operand: lane (l32, hh) keeps d = 16c + 8hh .. +7 of its query row for every 16-wide step c.
     u32x4 qf[D / 16];
-    {
-        const uint16_t *qp = p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2] + 8 * hh;
+    auto load_q = [&](int b_, int h_, int qt_) {
+        const int qrow_ = qt_ * (NW * 32) + wave * 32 + l32;
+        const uint16_t *qp = p.q + b_ * p.qs[0] + h_ * p.qs[1] + (int64_t)qrow_ * p.qs[2] + 8 * hh;
 #pragma unroll
         for (int c = 0; c < D / 16; c++) qf[c] = *(const u32x4 *)(qp + 16 * c);
-        // The scale (softmax scale / ln 2) goes into Q once, so that the S MFMAs deliver exp2 arguments.
+    };
+    // The scale (softmax scale / ln 2) goes into Q once, so that the S MFMAs deliver exp2 arguments.
+    auto scale_q = [&]() {
 #pragma unroll
         for (int c = 0; c < D / 16; c++)
 #pragma unroll
             for (int e = 0; e < 4; e++) qf[c][e] = E::scale2(qf[c][e], p.scale);
-    }
+    };
+    load_q(b, h, qt);
+    scale_q();
 
     // Online-softmax state of this lane's query row.  Exponentials are taken against a reference value m_ref
     // (exp2 units).  The S MFMAs start from the accumulator -m_ref (neg_m: the same value in all 16 registers,
@@ -187,7 +245,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
     // The Q tile's list (FULL entries, then PARTIAL entries) as first key columns, copied to LDS once:
     // loads issued after the first barrier cannot use the scalar cache, and a vector load of an index in
     // front of every chunk would put a full memory round trip on the critical path.
-    const bool list_in_lds = NE <= kListCap;
+    const bool list_in_lds = !PS && NE <= kListCap;
     if (list_in_lds) {
         for (int e = tid; e < NE; e += NW * 64) {
             const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
@@ -240,6 +298,54 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         entries_read(t, raw);
         entries_use(t, raw, col, valid, part);
     };
+    // Persistent workgroups keep the lists of two Q tiles in LDS (kPsListCap entries each), every entry with its
+    // kind in the top bits, padded with ABSENT entries to whole chunks:
+    //   bits 0..29 first key column, bit 30 PARTIAL, bit 31 ABSENT.
+    constexpr int NT = NW * 64;
+    constexpr int PER = kPsListCap / NT;  // list entries per thread
+    constexpr int kPartialBit = 1 << 30;
+    const int lbk_rt = MODE == 2 ? p.lbk : LBKC;
+    auto ps_list_issue = [&](int b_, int h_, int qt_, int F_, int P_, int(&lr)[PER]) {  // indices -> registers
+        const int32_t *f_ = p.full_ids + b_ * p.fis[0] + h_ * p.fis[1] + qt_ * p.fis[2];
+        const int32_t *p_ = p.part_ids + b_ * p.pis[0] + h_ * p.pis[1] + qt_ * p.pis[2];
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int e = tid + NT * i;
+            // slots past the count are read too (slot 0 of the row: always there) and flagged ABSENT on deposit
+            const int32_t *a = e < F_ ? f_ + (int64_t)e * p.fis[3]
+                                      : p_ + (int64_t)(e < F_ + P_ ? e - F_ : 0) * p.pis[3];
+            lr[i] = *a;
+        }
+    };
+    auto ps_list_deposit = [&](int F_, int P_, const int(&lr)[PER], int *dst) {  // registers -> LDS
+        const int ne = F_ + P_;
+        const int cnt = MODE == 2 ? (ne > 0 ? ne : 1) : chunks_of(ne) * EPC;
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int e = tid + NT * i;
+            if (e < cnt) dst[e] = e >= ne ? (int)0x80000000u : ((lr[i] << lbk_rt) | (e >= F_ ? kPartialBit : 0));
+        }
+    };
+    auto ps_entries_read = [&](const int *el, int t, int(&raw)[EPC]) {
+        if constexpr (MODE == 2) {
+            raw[0] = el[t >> (p.lbk - 6)];
+        } else {
+#pragma unroll
+            for (int j = 0; j < EPC; j++) raw[j] = el[t * EPC + j];
+        }
+    };
+    auto ps_entries_use = [&](int t, const int(&raw)[EPC], int(&col)[EPC], unsigned &valid, unsigned &part) {
+        valid = 0u;
+        part = 0u;
+#pragma unroll
+        for (int j = 0; j < EPC; j++) {
+            const int v = __builtin_amdgcn_readfirstlane(raw[j]);
+            col[j] = v & (kPartialBit - 1);
+            if constexpr (MODE == 2) col[j] += (t & ((1 << (p.lbk - 6)) - 1)) << 6;
+            if (v >= 0) valid |= 1u << j;
+            if (v & kPartialBit) part |= 1u << j;
+        }
+    };
 
     // Global -> LDS for one chunk, without passing through registers: 2*NLD direct loads per wave (piece 2i is
     // load i of K, piece 2i+1 load i of V).  A wave that issues them back to back sits at the issue stage until
@@ -286,7 +392,9 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
     // absent entries re-read the chunk's first entry and are discarded when the mask is applied.
     // No branches, eight independent loads, and no use of the loaded values here.
     constexpr int NMW = PK ? (MODE == 0 ? 4 : 2) : 8;  // mask words per lane and chunk
-    auto load_mask = [&](int t, const int(&col)[EPC], uint32_t(&mk)[NMW]) {
+    auto load_mask = [&](int t, const int(&col)[EPC], uint32_t(&mk)[NMW], const MaskSrc &ms) {
+        const uint8_t *const mrow = ms.mrow, *const prow = ms.prow;
+        const int F = ms.F, NE = ms.NE;
         if constexpr (PK) {
             // the row's bits of every entry of chunk t: one word (BK = 32), one halfword (BK = 16) per entry, or
             // the two words of the chunk's 64 keys (BK >= 64).  Entries that are not PARTIAL read slot 0.
@@ -391,7 +499,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
                     uint32_t w;
                     if constexpr (MODE == 0) w = word(2 * kb, 0xffffu) | (word(2 * kb + 1, 0xffffu) << 16);
                     else if constexpr (MODE == 1) w = word(kb, ~0u);
-                    else w = mk[kb];  // a chunk of a PARTIAL entry
+                    else w = (valid & 1u) ? mk[kb] : 0u;  // a chunk of a PARTIAL entry (or of an absent one)
                     w >>= sh4;  // this lane's keys are 8g + 4hh + jj
 #pragma unroll
                     for (int g = 0; g < 4; g++)
@@ -508,7 +616,196 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         for (int i = 0; i < NMW; i++) asm volatile("" ::"v"(mk[i]));
     };
 
-    if constexpr (PP) {
+    // O = acc / l (sparse_attn_kernel.py:144); rows that attended to nothing give 0.
+    auto store_o = [&]() {
+        const float l_tot = l32 < 16 ? acc_l[0] : acc_l[1];
+        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        uint16_t *orow = p.o + orow_off;
+#pragma unroll
+        for (int db = 0; db < D / 32; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const u32x2 w = {E::pack2(acc[db][4 * g] * inv, acc[db][4 * g + 1] * inv),
+                                 E::pack2(acc[db][4 * g + 2] * inv, acc[db][4 * g + 3] * inv)};
+                *(u32x2 *)(orow + 32 * db + 8 * g) = w;
+            }
+    };
+
+    if constexpr (PS) {
+        // Persistent loop.  Per Q tile of this workgroup's row, the pipeline is
+        //   two tiles ahead  its schedule entry is loaded;
+        //   one tile ahead   its list indices are loaded into registers (issued when the tile before it starts)
+        //                    and written to the free LDS list when that tile starts;
+        //   last chunk of the tile before: its first chunk is fetched into the free K/V stage and, once the
+        //                    last S phase is over, its queries are loaded over the old ones.
+        // Everything issued during a tile has landed by the time it is used: every chunk ends in vmcnt(0).
+        int *const el0 = reinterpret_cast<int *>(smem + NS * KBUF + NS * VBUF);
+        auto elist = [&](int which) -> int * { return el0 + which * kPsListCap; };
+        int lb = 0;  // LDS list of the tile at hand
+        int it = 0;  // its position in the row
+        bool has_nx = 1 < n_items, has_n2 = 2 < n_items;
+        int nx_bh = 0, nx_qt = 0, nx_F = 0, nx_P = 0;  // the next tile
+        int n2_bh = 0, n2_qt = 0, n2_F = 0, n2_P = 0;  // the one after
+        int lr[PER];
+        auto rfl = [](int x) { return __builtin_amdgcn_readfirstlane(x); };
+        ps_list_issue(b, h, qt, F, NE - F, lr);
+        ps_list_deposit(F, NE - F, lr, elist(0));
+        if (has_nx) {
+            const int4 e1 = sched_row[2];
+            nx_bh = rfl(e1.x), nx_qt = rfl(e1.y), nx_F = rfl(e1.z), nx_P = rfl(e1.w);
+            ps_list_issue(nx_bh >> 16, nx_bh & 0xffff, nx_qt, nx_F, nx_P, lr);
+            ps_list_deposit(nx_F, nx_P, lr, elist(1));
+        }
+        if (has_n2) {
+            const int4 e2 = sched_row[3];
+            n2_bh = rfl(e2.x), n2_qt = rfl(e2.y), n2_F = rfl(e2.z), n2_P = rfl(e2.w);
+            ps_list_issue(n2_bh >> 16, n2_bh & 0xffff, n2_qt, n2_F, n2_P, lr);  // stays in registers for now
+        }
+        int4 e3 = 3 < n_items ? sched_row[4] : int4{0, 0, 0, 0};
+
+        int col[EPC], coln[EPC];
+        unsigned valid, part;
+        uint32_t mk[2][NMW] = {};
+        bool sp[2] = {false, false};
+        unsigned vl[2] = {0u, 0u}, pt[2] = {0u, 0u};
+        constexpr unsigned ALL = (1u << EPC) - 1u;
+        StagePlan pl;
+        int raw[EPC];
+        __syncthreads();  // the lists in LDS are complete
+        // first chunk of the first tile, and the look-ahead state of a tile that starts at the parity-0 stage:
+        // `pl`, coln, sp/vl/pt[1] describe chunk 1, raw holds the entries of chunk 2 (clamped to the last chunk)
+        ps_entries_read(elist(0), 0, raw);
+        ps_entries_use(0, raw, col, valid, part);
+        stage_chunk(0, col);
+        sp[0] = part != 0u || valid != ALL;
+        vl[0] = valid;
+        pt[0] = part;
+        if (sp[0]) load_mask(0, col, mk[0], MaskSrc{mrow, prow, F, NE});
+        ps_entries_read(elist(0), 1 < T ? 1 : 0, raw);
+        ps_entries_use(1 < T ? 1 : 0, raw, coln, valid, part);
+        sp[1] = 1 < T && (part != 0u || valid != ALL);
+        vl[1] = valid;
+        pt[1] = part;
+        plan_chunk(coln, pl);
+        ps_entries_read(elist(0), 2 < T ? 2 : T - 1, raw);
+#pragma unroll
+        for (int c = 0; c < D / 16; c++) asm volatile("" ::"v"(qf[c]));
+        settle(mk[0]);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+
+        int tc = 0;
+        bool done = false;
+        while (!done) {
+            static_for<2>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                constexpr int cur = j & 1, nxt = cur ^ 1;
+                if (done) return;
+                const bool last = tc == T - 1;
+                const bool cross = last && has_nx;  // the chunk fetched now is the first one of the next tile
+                const bool fetch = !last || has_nx;
+                MaskSrc msn{mrow, prow, F, NE};
+                const int nb_ = nx_bh >> 16, nh_ = nx_bh & 0xffff;
+                if (cross) {
+                    int rx[EPC];
+                    ps_entries_read(elist(lb ^ 1), 0, rx);
+                    ps_entries_use(0, rx, coln, valid, part);
+                    const uint16_t *kn = p.k + nb_ * p.ks[0] + nh_ * p.ks[1];
+                    const uint16_t *vn = p.v + nb_ * p.vs[0] + nh_ * p.vs[1];
+#pragma unroll
+                    for (int e = 0; e < EPC; e++) {
+                        pl.kp[e] = kn + (int64_t)coln[e] * p.ks[2];
+                        pl.vp[e] = vn + (int64_t)coln[e] * p.vs[2];
+                    }
+                    sp[nxt] = part != 0u || valid != ALL;
+                    vl[nxt] = valid;
+                    pt[nxt] = part;
+                    if (sp[nxt]) msn = mask_src_of(nb_, nh_, nx_qt, nx_F, nx_F + nx_P);
+                }
+                if (sp[nxt]) load_mask(cross ? 0 : tc + 1, coln, mk[nxt], msn);
+                f32x16 s[2];
+                phase_s(jc, s, std::integral_constant<int, nxt>{}, fetch, pl);
+                if (cross) load_q(nb_, nh_, nx_qt);  // the old queries have done their last S phase
+                const int t2 = tc + 2 < T ? tc + 2 : T - 1, t3 = tc + 3 < T ? tc + 3 : T - 1;
+                int col2[EPC];
+                unsigned valid2 = 0u, part2 = 0u;
+                StagePlan pl2;
+                const int *const el = elist(lb);
+                phase_pv(jc, s, sp[cur], vl[cur], pt[cur], mk[cur], [&](int bb, int nb) {
+                    const int per = (2 * EPC + nb - 1) / nb;  // plan entries per bundle
+                    if (bb == 0) ps_entries_use(t2, raw, col2, valid2, part2);
+#pragma unroll
+                    for (int i = bb * per; i < (bb + 1) * per && i < 2 * EPC; i++) {
+                        if (i & 1) pl2.vp[i >> 1] = vbase + (int64_t)col2[i >> 1] * p.vs[2];
+                        else pl2.kp[i >> 1] = kbase + (int64_t)col2[i >> 1] * p.ks[2];
+                    }
+                    if (bb == nb - 1) ps_entries_read(el, t3, raw);
+                });
+                pl = pl2;
+#pragma unroll
+                for (int e = 0; e < EPC; e++) coln[e] = col2[e];
+                const bool sp2 = tc + 2 < T && (part2 != 0u || valid2 != ALL);
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the fetched chunk and its mask words have landed
+                settle(mk[nxt]);  // on every path: the compiler cannot tell that loads and uses share a condition
+                // same for the queries (new ones are loaded when `cross`): accounted for here on every path, so that
+                // the S phases of the loop carry no wait for them
+#pragma unroll
+                for (int c = 0; c < D / 16; c++) asm volatile("" ::"v"(qf[c]));
+                sp[cur] = sp2;
+                vl[cur] = valid2;
+                pt[cur] = part2;
+                if (!last) {
+                    tc++;
+                    __syncthreads();
+                    return;
+                }
+                // ---- the tile is finished --------------------------------------------------------------
+                store_o();
+                if (!has_nx) {
+                    done = true;
+                    return;
+                }
+                set_item(nb_, nh_, nx_qt, nx_F, nx_P);
+                lb ^= 1;
+                it++;
+                tc = 0;
+                // the list that waited in registers goes to the LDS list the finished tile used
+                if (has_n2) ps_list_deposit(n2_F, n2_P, lr, elist(lb ^ 1));
+                has_nx = has_n2;
+                nx_bh = n2_bh, nx_qt = n2_qt, nx_F = n2_F, nx_P = n2_P;
+                has_n2 = it + 2 < n_items;
+                if (has_n2) {
+                    n2_bh = rfl(e3.x), n2_qt = rfl(e3.y), n2_F = rfl(e3.z), n2_P = rfl(e3.w);
+                    ps_list_issue(n2_bh >> 16, n2_bh & 0xffff, n2_qt, n2_F, n2_P, lr);
+                }
+                if (it + 3 < n_items) e3 = sched_row[1 + it + 3];
+                // fresh softmax state; the new queries were loaded during the last P.V phase
+                m_ref = 0.f;
+                raise_above = -3.0e38f;
+#pragma unroll
+                for (int i = 0; i < 16; i++) neg_m[i] = 0.f;
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc_l[i] = 0.f;
+#pragma unroll
+                for (int db = 0; db < D / 32; db++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) acc[db][i] = 0.f;
+                scale_q();
+                // look-ahead state of the new tile; its chunk 0 sits in stage nxt, so chunk 1 goes to stage cur
+                const int *const eln = elist(lb);
+                int rx[EPC];
+                ps_entries_read(eln, 1 < T ? 1 : 0, rx);
+                ps_entries_use(1 < T ? 1 : 0, rx, coln, valid, part);
+                sp[cur] = 1 < T && (part != 0u || valid != ALL);
+                vl[cur] = valid;
+                pt[cur] = part;
+                plan_chunk(coln, pl);
+                ps_entries_read(eln, 2 < T ? 2 : T - 1, raw);
+                __syncthreads();
+            });
+        }
+        return;
+    } else if constexpr (PP) {
         // Ping-pong schedule.  Every wave runs  barrier | S phase | barrier | P.V phase  per chunk; waves 4..7
         // enter the sequence one barrier later than waves 0..3, so between two barriers one wave of each SIMD
         // issues the MFMA-only S phase while the other does softmax and P.V, and the matrix unit always has a
@@ -531,7 +828,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
             sp[0] = part != 0u || valid != ALL;
             vl[0] = valid;
             pt[0] = part;
-            if (sp[0]) load_mask(0, col, mk[0]);
+            if (sp[0]) load_mask(0, col, mk[0], MaskSrc{mrow, prow, F, NE});
 #pragma unroll
             for (int j = 0; j < EPC; j++) coln[j] = col[j];
             if (1 < T) {
@@ -542,7 +839,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
             for (int c = 0; c < D / 16; c++) asm volatile("" ::"v"(qf[c]));
             int raw[EPC] = {};  // list entries of the chunk after next, read ahead
             if (2 < T) entries_read(2, raw);
-            if (sp[0]) settle(mk[0]);
+            settle(mk[0]);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
             if (late) __syncthreads();
@@ -554,14 +851,14 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
                     if (tc < T) {
                         // own pieces of chunk tc have landed; chunk tc+1 may be in flight
                         wait_vm_at_most((tc + 1 < T ? tc + 1 : T - 1) - tc, kOpsPerChunk);
-                        if (sp[cur]) settle(mk[cur]);
+                        if (sp[cur]) settle(mk[cur]);  // (the compiler's wait for them takes the chunk in flight along)
                         __syncthreads();
                         sp[nxt] = false;
                         if (tc + 1 < T) {  // coln: entries of chunk tc+1
                             sp[nxt] = partn != 0u || validn != ALL;
                             vl[nxt] = validn;
                             pt[nxt] = partn;
-                            if (sp[nxt]) load_mask(tc + 1, coln, mk[nxt]);
+                            if (sp[nxt]) load_mask(tc + 1, coln, mk[nxt], MaskSrc{mrow, prow, F, NE});
                         }
                         const bool fetch = tc + 2 < T;
                         if (fetch) {
@@ -596,7 +893,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         sp[0] = part != 0u || valid != ALL;
         vl[0] = valid;
         pt[0] = part;
-        if (sp[0]) load_mask(0, col, mk[0]);
+        if (sp[0]) load_mask(0, col, mk[0], MaskSrc{mrow, prow, F, NE});
         chunk_entries(1 < T ? 1 : 0, coln, valid, part);
         sp[1] = 1 < T && (part != 0u || valid != ALL);
         vl[1] = valid;
@@ -606,7 +903,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         entries_read(2 < T ? 2 : T - 1, raw);
 #pragma unroll
         for (int c = 0; c < D / 16; c++) asm volatile("" ::"v"(qf[c]));
-        if (sp[0]) settle(mk[0]);
+        settle(mk[0]);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         // Two chunks per trip so that the LDS stage is a compile-time constant.  Iteration tc computes chunk tc
@@ -620,7 +917,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
                 const int tc = t + j;
                 if (tc < T) {
                     const bool fetch = tc + 1 < T;
-                    if (sp[nxt]) load_mask(tc + 1, coln, mk[nxt]);
+                    if (sp[nxt]) load_mask(tc + 1, coln, mk[nxt], MaskSrc{mrow, prow, F, NE});
                     f32x16 s[2];
                     phase_s(jc, s, std::integral_constant<int, nxt>{}, fetch, pl);
                     const int t2 = tc + 2 < T ? tc + 2 : T - 1, t3 = tc + 3 < T ? tc + 3 : T - 1;
@@ -643,7 +940,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
                     // chunk tc+2 will be computed from the slot of chunk tc
                     const bool sp2 = tc + 2 < T && (part2 != 0u || valid2 != ALL);
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // chunk tc+1 and its mask words have landed
-                    if (sp[nxt]) settle(mk[nxt]);
+                    settle(mk[nxt]);  // on every path: the compiler cannot tell that loads and uses share a condition
                     sp[cur] = sp2;
                     vl[cur] = valid2;
                     pt[cur] = part2;
@@ -653,26 +950,16 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         }
     }
 
-    // Epilogue: O = acc / l (sparse_attn_kernel.py:144); rows that attended to nothing give 0.
-    const float l_tot = l32 < 16 ? acc_l[0] : acc_l[1];
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    uint16_t *orow = p.o + b * p.os[0] + h * p.os[1] + (int64_t)qrow * p.os[2] + 4 * hh;
-#pragma unroll
-    for (int db = 0; db < D / 32; db++)
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const u32x2 w = {E::pack2(acc[db][4 * g] * inv, acc[db][4 * g + 1] * inv),
-                             E::pack2(acc[db][4 * g + 2] * inv, acc[db][4 * g + 3] * inv)};
-            *(u32x2 *)(orow + 32 * db + 8 * g) = w;
-        }
+    store_o();
 }
 
-template <int DT, int D, int NW, int MODE, bool PK>
+template <int DT, int D, int NW, int MODE, bool PK, bool PS>
 hipError_t launch_one(const FwdParams &p, hipStream_t stream) {
     // Eight waves fill a CU's register file on their own, so that workgroup can have most of the LDS: 4 stages.
     constexpr int NS = NW == 8 ? 4 : 2;
-    constexpr int smem = 2 * NS * 64 * D * 2 + kListCap * 4;  // NS stages of 64 rows for K and for V + the list
-    auto kern = sparse_fwd_kernel<DT, D, NW, MODE, NS, NW == 8, PK>;
+    static_assert(kListCap == 2 * kPsListCap, "one long list or two short ones in the same LDS");
+    constexpr int smem = 2 * NS * 64 * D * 2 + kListCap * 4;  // NS stages of 64 rows for K and for V + the list(s)
+    auto kern = sparse_fwd_kernel<DT, D, NW, MODE, NS, NW == 8, PK, PS>;
     static bool attr_set = false;  // benign race: every thread sets the same value
     if (!attr_set) {
         const hipError_t e =
@@ -680,38 +967,41 @@ hipError_t launch_one(const FwdParams &p, hipStream_t stream) {
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    const unsigned grid = (unsigned)p.nQ * (unsigned)p.B * (unsigned)p.H;
+    const unsigned grid = PS ? (unsigned)p.sched_G : (unsigned)p.nQ * (unsigned)p.B * (unsigned)p.H;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), smem, stream, p);
     return hipGetLastError();
 }
 
-template <int DT, int D, int NW, bool PK>
+template <int DT, int D, int NW, bool PK, bool PS>
 hipError_t launch_mode(const FwdParams &p, hipStream_t stream) {
-    if (p.BK == 16) return launch_one<DT, D, NW, 0, PK>(p, stream);
-    if (p.BK == 32) return launch_one<DT, D, NW, 1, PK>(p, stream);
-    return launch_one<DT, D, NW, 2, PK>(p, stream);
+    if (p.BK == 16) return launch_one<DT, D, NW, 0, PK, PS>(p, stream);
+    if (p.BK == 32) return launch_one<DT, D, NW, 1, PK, PS>(p, stream);
+    return launch_one<DT, D, NW, 2, PK, PS>(p, stream);
 }
 
-template <int DT, int D, bool PK>
+template <int DT, int D, bool PK, bool PS>
 hipError_t launch_bq(const FwdParams &p, int BQ, hipStream_t stream) {
     switch (BQ) {
-        case 32: return launch_mode<DT, D, 1, PK>(p, stream);
-        case 64: return launch_mode<DT, D, 2, PK>(p, stream);
-        case 128: return launch_mode<DT, D, 4, PK>(p, stream);
-        case 256: return launch_mode<DT, D, 8, PK>(p, stream);
+        case 32: return launch_mode<DT, D, 1, PK, PS>(p, stream);
+        case 64: return launch_mode<DT, D, 2, PK, PS>(p, stream);
+        case 128: return launch_mode<DT, D, 4, PK, PS>(p, stream);
+        case 256:
+            if constexpr (PS) return hipErrorInvalidValue;  // 8-wave workgroups are not persistent
+            else return launch_mode<DT, D, 8, PK, false>(p, stream);
         default: return hipErrorInvalidValue;
     }
 }
 
 }  // namespace
 
-// Every kernel for one element type and one source of the PARTIAL tiles' mask entries.  Each combination is
-// instantiated in a translation unit of its own (sparse_fwd_inst.hip compiled with SA_FWD_DT / SA_FWD_PK).
-template <int DT, bool PK>
+// Every kernel for one element type, one source of the PARTIAL tiles' mask entries and one way of handing out
+// Q tiles.  Each combination is instantiated in a translation unit of its own (sparse_fwd_inst.hip compiled
+// with SA_FWD_DT / SA_FWD_PK / SA_FWD_PS).
+template <int DT, bool PK, bool PS>
 hipError_t launch_fwd_variant(const FwdParams &p, int D, int BQ, hipStream_t stream) {
     switch (D) {
-        case 64: return launch_bq<DT, 64, PK>(p, BQ, stream);
-        case 128: return launch_bq<DT, 128, PK>(p, BQ, stream);
+        case 64: return launch_bq<DT, 64, PK, PS>(p, BQ, stream);
+        case 128: return launch_bq<DT, 128, PK, PS>(p, BQ, stream);
         default: return hipErrorInvalidValue;
     }
 }

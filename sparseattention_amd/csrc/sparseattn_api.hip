@@ -138,13 +138,37 @@ int sa_mask_classify(const uint8_t *mask, const int64_t mask_strides[4], int B, 
 
 namespace {
 
+// Workgroups the persistent forward launches on the current device (2 per compute unit, a multiple of 8, at
+// most 512), entries per schedule row, and the bytes of the schedule; 0 when there is no persistent kernel for
+// the problem or no device.
+size_t schedule_shape(int B, int H, int Sq, int Sk, int BQ, int BK, int *G_out, int *R_out) {
+    if (B <= 0 || H <= 0 || Sq <= 0 || Sk <= 0 || BQ <= 0 || BK <= 0 || Sq % BQ || Sk % BK) return 0;
+    if (BQ != 32 && BQ != 64 && BQ != 128) return 0;
+    if (log2_exact(BK) < 4 || Sk / BK > 1024 || B >= 32768 || H >= 65536) return 0;
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    int G = 2 * cus;
+    if (G > 512) G = 512;
+    G &= ~7;
+    if (G < 8) return 0;
+    const int64_t N = (int64_t)B * H * (Sq / BQ);
+    const int64_t NX = (N + 7) / 8;
+    const int64_t R = (NX + G / 8 - 1) / (G / 8);
+    if (R > 0x3fffffff) return 0;
+    if (G_out) *G_out = G;
+    if (R_out) *R_out = (int)R;
+    return (size_t)G * (size_t)(R + 1) * 16;
+}
+
 int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4], const void *v,
                  const int64_t v_strides[4], void *o, const int64_t o_strides[4], const uint8_t *mask,
                  const int64_t mask_strides[4], const int32_t *full_ids, const int64_t full_ids_strides[4],
                  const int32_t *full_lens, const int64_t full_lens_strides[3], const int32_t *part_ids,
                  const int64_t part_ids_strides[4], const int32_t *part_lens, const int64_t part_lens_strides[3],
-                 const uint8_t *packed, const int64_t packed_strides[2], bool use_packed, int B, int H, int Sq, int Sk,
-                 int D, int BQ, int BK, int dtype, float sm_scale_log2, void *stream) {
+                 const uint8_t *packed, const int64_t packed_strides[2], bool use_packed, const int32_t *schedule,
+                 size_t schedule_bytes, int B, int H, int Sq, int Sk, int D, int BQ, int BK, int dtype,
+                 float sm_scale_log2, void *stream) {
     g_error[0] = 0;
     if (!q || !k || !v || !o || !q_strides || !k_strides || !v_strides || !o_strides || !full_ids ||
         !full_ids_strides || !full_lens || !full_lens_strides || !part_ids || !part_ids_strides || !part_lens ||
@@ -205,6 +229,18 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
     fp.pks[0] = use_packed ? packed_strides[0] : 0;
     fp.pks[1] = use_packed ? packed_strides[1] : 0;
     fp.nK = Sk / BK;
+    fp.sched = nullptr;
+    if (schedule) {
+        int G = 0, R = 0;
+        const size_t want = schedule_shape(B, H, Sq, Sk, BQ, BK, &G, &R);
+        if (want != 0 && want == schedule_bytes) {
+            if (!aligned(schedule, 16))
+                return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd_ex: schedule needs a 16-byte aligned base");
+            fp.sched = schedule;
+            fp.sched_G = G;
+            fp.sched_R = R;
+        }
+    }
     fp.B = B;
     fp.H = H;
     fp.Sq = Sq;
@@ -250,29 +286,68 @@ int sa_sparse_attention_fwd(const void *q, const int64_t q_strides[4], const voi
                             int dtype, float sm_scale_log2, void *stream) {
     return forward_impl(q, q_strides, k, k_strides, v, v_strides, o, o_strides, mask, mask_strides, full_ids,
                         full_ids_strides, full_lens, full_lens_strides, part_ids, part_ids_strides, part_lens,
-                        part_lens_strides, nullptr, nullptr, false, B, H, Sq, Sk, D, BQ, BK, dtype, sm_scale_log2,
-                        stream);
+                        part_lens_strides, nullptr, nullptr, false, nullptr, 0, B, H, Sq, Sk, D, BQ, BK, dtype,
+                        sm_scale_log2, stream);
 }
 
-int sa_sparse_attention_fwd_packed(const void *q, const int64_t q_strides[4], const void *k,
-                                   const int64_t k_strides[4], const void *v, const int64_t v_strides[4], void *o,
-                                   const int64_t o_strides[4], const uint8_t *mask, const int64_t mask_strides[4],
-                                   const int32_t *full_ids, const int64_t full_ids_strides[4],
-                                   const int32_t *full_lens, const int64_t full_lens_strides[3],
-                                   const int32_t *part_ids, const int64_t part_ids_strides[4],
-                                   const int32_t *part_lens, const int64_t part_lens_strides[3],
-                                   const uint8_t *packed, const int64_t packed_strides[2], int B, int H, int Sq,
-                                   int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2, void *stream) {
-    if (packed && packed_strides) {
-        if ((B > 1 && packed_strides[0] % 4) || (H > 1 && packed_strides[1] % 4) || !aligned(packed, 4)) {
-            g_error[0] = 0;
-            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd_packed: packed needs a 4-byte aligned base and plane strides");
-        }
+int sa_sparse_attention_fwd_ex(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                               const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
+                               const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
+                               const int64_t full_ids_strides[4], const int32_t *full_lens,
+                               const int64_t full_lens_strides[3], const int32_t *part_ids,
+                               const int64_t part_ids_strides[4], const int32_t *part_lens,
+                               const int64_t part_lens_strides[3], const uint8_t *packed,
+                               const int64_t packed_strides[2], const int32_t *schedule, size_t schedule_bytes, int B,
+                               int H, int Sq, int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2,
+                               void *stream) {
+    const bool use_packed = packed != nullptr;
+    if (use_packed) {
+        g_error[0] = 0;
+        if (!packed_strides) return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd_ex: null pointer argument (packed_strides)");
+        if ((B > 1 && packed_strides[0] % 4) || (H > 1 && packed_strides[1] % 4) || !aligned(packed, 4))
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd_ex: packed needs a 4-byte aligned base and plane strides");
     }
     return forward_impl(q, q_strides, k, k_strides, v, v_strides, o, o_strides, mask, mask_strides, full_ids,
                         full_ids_strides, full_lens, full_lens_strides, part_ids, part_ids_strides, part_lens,
-                        part_lens_strides, packed, packed_strides, true, B, H, Sq, Sk, D, BQ, BK, dtype,
-                        sm_scale_log2, stream);
+                        part_lens_strides, packed, packed_strides, use_packed, schedule, schedule_bytes, B, H, Sq, Sk,
+                        D, BQ, BK, dtype, sm_scale_log2, stream);
+}
+
+size_t sa_fwd_schedule_bytes(int B, int H, int Sq, int Sk, int BQ, int BK) {
+    return schedule_shape(B, H, Sq, Sk, BQ, BK, nullptr, nullptr);
+}
+
+int sa_fwd_schedule(const int32_t *full_lens, const int64_t full_lens_strides[3], const int32_t *part_lens,
+                    const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int BQ, int BK,
+                    int32_t *schedule, size_t schedule_bytes, void *stream) {
+    g_error[0] = 0;
+    if (!full_lens || !full_lens_strides || !part_lens || !part_lens_strides || !schedule)
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_fwd_schedule: null pointer argument");
+    if (const int rc = check_tiling(B, H, Sq, Sk, BQ, BK)) return rc;
+    int G = 0, R = 0;
+    const size_t want = schedule_shape(B, H, Sq, Sk, BQ, BK, &G, &R);
+    if (want == 0)
+        return fail(SA_ERR_UNSUPPORTED, "sa_fwd_schedule: no persistent forward for BLOCK_Q %d, BLOCK_K %d, Sk %d (BLOCK_Q 32/64/128, BLOCK_K a power of two >= 16, Sk/BLOCK_K <= 1024), or no device", BQ, BK, Sk);
+    if (schedule_bytes != want)
+        return fail(SA_ERR_WORKSPACE, "sa_fwd_schedule: schedule of %zu bytes required, %zu given", want, schedule_bytes);
+    if (!aligned(schedule, 16)) return fail(SA_ERR_UNSUPPORTED, "sa_fwd_schedule: schedule needs a 16-byte aligned base");
+    sa::ScheduleParams sp{};
+    sp.full_lens = full_lens;
+    sp.part_lens = part_lens;
+    for (int i = 0; i < 3; i++) {
+        sp.fls[i] = full_lens_strides[i];
+        sp.pls[i] = part_lens_strides[i];
+    }
+    sp.B = B;
+    sp.H = H;
+    sp.nQ = Sq / BQ;
+    sp.G = G;
+    sp.R = R;
+    sp.lbk = log2_exact(BK);
+    sp.sched = schedule;
+    const hipError_t e = sa::launch_schedule(sp, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_fwd_schedule: launch failed: %s", hipGetErrorString(e));
+    return SA_OK;
 }
 
 size_t sa_mask_pack_partial_bytes(const int64_t mask_strides[4], int B, int H, int Sq, int Sk, int BQ, int BK) {

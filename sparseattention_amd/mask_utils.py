@@ -27,6 +27,11 @@ class MaskMetadata:
     the PARTIAL tiles at one bit each.  ``packed_masks[b,h,qt,slot]`` belongs to KV tile
     ``masked_kv_ids[b,h,qt,slot]``: rows first, entry (r, c) in bit ``c & 7`` of byte ``(r*BK + c) >> 3``.
     When present, :func:`sparse_attention` reads these bits and never touches the bool mask.
+
+    ``schedule`` is the second addition (optional, default None): int32 [workgroups, rounds + 1, 4], which Q tiles
+    each of the forward's persistent workgroups processes, in order (entry 0 of a row: the count; then
+    ``((b << 16) | h, qt, unmasked_len, masked_len)`` per tile).  It depends on the counts, on B and H and on
+    the device; without it the forward launches one workgroup per Q tile.
     """
 
     unmasked_kv_ids: torch.Tensor
@@ -34,6 +39,7 @@ class MaskMetadata:
     masked_kv_ids: torch.Tensor
     masked_lens: torch.Tensor
     packed_masks: Optional[torch.Tensor] = None
+    schedule: Optional[torch.Tensor] = None
 
 
 def _check_mask(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int):
@@ -75,8 +81,8 @@ def compute_mask_slow(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int) -> MaskMet
     return MaskMetadata(fid, fl, pid, pl)
 
 
-def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int,
-                        pack_partial: Optional[bool] = None) -> MaskMetadata:
+def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int, pack_partial: Optional[bool] = None,
+                        schedule: bool = False) -> MaskMetadata:
     """Classify the mask's tiles on the GPU (replaces mask_utils.py:85-107).
 
     ``mask``: bool [B,H,Sq,Sk] on a ROCm device, any strides.  Dimensions that are broadcast in
@@ -86,6 +92,10 @@ def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int,
 
     ``pack_partial``: also fill ``MaskMetadata.packed_masks`` (Sq*Sk/8 bytes per distinct mask plane).
     Default: whenever BLOCK_K is a multiple of 8; ``False`` gives exactly the reference's four tensors.
+    ``schedule``: also fill ``MaskMetadata.schedule`` (needs BLOCK_Q 32/64/128, BLOCK_K a power of two >= 16
+    and at most 1024 KV tiles per row).  Off by default: measured on MI355X, persistent workgroups win when the
+    lists are short (a few hundred keys per Q tile) and lose a few percent to the hardware dispatcher when
+    they are long, because a static hand-out cannot follow the uneven pace of the workgroups that share a CU.
     """
     B, H, Sq, Sk = _check_mask(mask, BLOCK_Q, BLOCK_K)
     if not mask.is_cuda:
@@ -130,7 +140,20 @@ def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int,
             )
             _native.check(rc)
             packed = packed.expand(B, H, nQ, nK, BLOCK_Q * BLOCK_K // 8)
-    return MaskMetadata(fid, fl, pid, pl, packed)
+        sched = None
+        if schedule:
+            nbytes = int(lib.sa_fwd_schedule_bytes(B, H, Sq, Sk, BLOCK_Q, BLOCK_K))
+            if nbytes == 0:
+                raise ValueError(f"no persistent forward for BLOCK_Q={BLOCK_Q}, BLOCK_K={BLOCK_K}, Sk={Sk}")
+            if nbytes:
+                sched = torch.empty(nbytes // 4, dtype=torch.int32, device=dev)
+                rc = lib.sa_fwd_schedule(fl.data_ptr(), _native.strides(fl.stride()), pl.data_ptr(),
+                                         _native.strides(pl.stride()), B, H, Sq, Sk, BLOCK_Q, BLOCK_K,
+                                         sched.data_ptr(), nbytes, torch.cuda.current_stream(dev).cuda_stream)
+                _native.check(rc)
+                G = min(2 * torch.cuda.get_device_properties(dev).multi_processor_count, 512) & ~7
+                sched = sched.view(G, nbytes // (16 * G), 4)
+    return MaskMetadata(fid, fl, pid, pl, packed, sched)
 
 
 # Tile sizes tried by select_block_sizes, and what one executed mask entry costs at each BLOCK_Q relative to

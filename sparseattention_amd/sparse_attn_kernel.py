@@ -61,6 +61,10 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
             raise ValueError(f"mask_metadata.packed_masks: expected uint8 {shape} on {q.device} with contiguous "
                              f"tiles, got {packed.dtype} {tuple(packed.shape)} strides {packed.stride()}")
 
+    sched = getattr(mask_metadata, "schedule", None)
+    if sched is not None and (sched.dtype != torch.int32 or sched.device != q.device or not sched.is_contiguous()):
+        raise ValueError("mask_metadata.schedule: expected a contiguous int32 tensor on q's device")
+
     qc, kc, vc = _kernel_ready(q), _kernel_ready(k), _kernel_ready(v)
     o = torch.empty_like(qc)
     lib = _native.load()
@@ -72,8 +76,11 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
                   pid.data_ptr(), S(pid.stride()), pl.data_ptr(), S(pl.stride()))
         tail = (B, H, Sq, Sk, D, int(BLOCK_Q), int(BLOCK_K), _DTYPES[q.dtype], sm_scale,
                 torch.cuda.current_stream(q.device).cuda_stream)
-        if packed is not None:
-            rc = lib.sa_sparse_attention_fwd_packed(*common, packed.data_ptr(), S(packed.stride()[:2]), *tail)
+        sched = getattr(mask_metadata, "schedule", None)
+        if packed is not None or sched is not None:
+            pk = (packed.data_ptr(), S(packed.stride()[:2])) if packed is not None else (None, None)
+            sc = (sched.data_ptr(), sched.numel() * 4) if sched is not None else (None, 0)
+            rc = lib.sa_sparse_attention_fwd_ex(*common, *pk, *sc, *tail)
         else:
             rc = lib.sa_sparse_attention_fwd(*common, *tail)
     _native.check(rc)

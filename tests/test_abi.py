@@ -122,23 +122,43 @@ def test_pack_rejects_bad_arguments_and_sizes_its_buffer():
     assert "overlap" in last_error()
 
 
-def test_packed_forward_rejects_bad_arguments():
+def test_extended_forward_rejects_bad_arguments():
     lib = _native.load()
     qs = _native.strides((256 * 128, 256 * 128, 128, 1))
 
-    def call(packed=FAKE, ps=_native.strides((0, 0)), mask=None, BK=32, B=1):
-        return lib.sa_sparse_attention_fwd_packed(FAKE, qs, FAKE, qs, FAKE, qs, FAKE, qs, mask, None, FAKE, I4, FAKE,
-                                                  S3, FAKE, I4, FAKE, S3, packed, ps, B, 1, 256, 256, 128, 128, BK, 0,
-                                                  0.1, None)
+    def call(packed=FAKE, ps=_native.strides((0, 0)), mask=None, BK=32, B=1, sched=None, sched_bytes=0):
+        return lib.sa_sparse_attention_fwd_ex(FAKE, qs, FAKE, qs, FAKE, qs, FAKE, qs, mask, None, FAKE, I4, FAKE, S3,
+                                              FAKE, I4, FAKE, S3, packed, ps, sched, sched_bytes, B, 1, 256, 256, 128,
+                                              128, BK, 0, 0.1, None)
 
-    assert call(packed=None) == _native.SA_ERR_INVALID_ARGUMENT and "packed" in last_error()
+    # neither a mask nor packed bits
+    assert call(packed=None) == _native.SA_ERR_INVALID_ARGUMENT and "mask" in last_error()
     assert call(ps=None) == _native.SA_ERR_INVALID_ARGUMENT
     assert call(packed=FAKE + 2) == _native.SA_ERR_UNSUPPORTED and "aligned" in last_error()
     assert call(B=2, ps=_native.strides((6, 0))) == _native.SA_ERR_UNSUPPORTED
     assert call(BK=8) == _native.SA_ERR_UNSUPPORTED and "BLOCK_K" in last_error()
-    # the plain entry point still insists on a mask
+    # the plain entry point insists on a mask
     assert lib.sa_sparse_attention_fwd(FAKE, qs, FAKE, qs, FAKE, qs, FAKE, qs, None, None, FAKE, I4, FAKE, S3, FAKE, I4,
                                        FAKE, S3, 1, 1, 256, 256, 128, 128, 32, 0, 0.1, None) == _native.SA_ERR_INVALID_ARGUMENT
+
+
+def test_schedule_rejects_bad_arguments():
+    lib = _native.load()
+
+    def call(fl=FAKE, sched=FAKE, nbytes=16, Sq=256, BQ=128, BK=32):
+        return lib.sa_fwd_schedule(fl, S3, FAKE, S3, 1, 1, Sq, 256, BQ, BK, sched, nbytes, None)
+
+    assert call(fl=None) == _native.SA_ERR_INVALID_ARGUMENT and "null" in last_error()
+    assert call(sched=None) == _native.SA_ERR_INVALID_ARGUMENT
+    assert call(Sq=200) == _native.SA_ERR_INVALID_ARGUMENT
+    # tile sizes without a persistent kernel (and, without a GPU, every size): unsupported, nothing launched
+    assert call(BQ=256) == _native.SA_ERR_UNSUPPORTED and "persistent" in last_error()
+    assert call(BK=8) == _native.SA_ERR_UNSUPPORTED
+    assert lib.sa_fwd_schedule_bytes(1, 1, 256, 256, 256, 32) == 0
+    assert lib.sa_fwd_schedule_bytes(1, 1, 256, 256, 100, 32) == 0
+    if not torch.cuda.is_available():
+        assert lib.sa_fwd_schedule_bytes(1, 1, 256, 256, 128, 32) == 0
+        assert call() == _native.SA_ERR_UNSUPPORTED
 
 
 def test_python_wrappers_refuse_to_run_without_a_gpu_tensor():
