@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define SA_ABI_VERSION 3
+#define SA_ABI_VERSION 4
 
 enum sa_status {
     SA_OK = 0,
@@ -51,6 +51,11 @@ enum sa_status {
 enum sa_dtype {
     SA_DTYPE_BF16 = 0,
     SA_DTYPE_FP16 = 1
+};
+
+enum sa_schedule_mode {
+    SA_SCHEDULE_PERSISTENT = 0, /* as many workgroups as the device holds at once, each walks many Q tiles */
+    SA_SCHEDULE_PAIRS = 1       /* one workgroup per two Q tiles, a long list with a short one under causal masks */
 };
 
 /* ABI version of the loaded library (== SA_ABI_VERSION it was built with). */
@@ -147,22 +152,27 @@ int sa_mask_pack_partial(const uint8_t *mask, const int64_t mask_strides[4], int
                          const int64_t packed_strides[2], void *stream);
 
 /*
- * Schedule of the forward's persistent workgroups.  No counterpart in the reference, whose grid is one program
- * per Q tile (sparse_attn_kernel.py:167): here a grid that fills the device once walks over the Q tiles, so that
- * the start-up latencies of a workgroup (arguments, counts, lists, first K/V tiles) are not paid per Q tile, and
- * the tiles are dealt out by their known cost (the list lengths) instead of in launch order.
+ * Schedule of the forward: which Q tiles a workgroup processes, in order.  No counterpart in the reference, whose
+ * grid is one program per Q tile (sparse_attn_kernel.py:167).  A workgroup that walks several Q tiles runs one
+ * chunk stream across them: the next tile's first K/V rows, its queries and its list are on their way while the
+ * current tile is computed, so the start-up latencies of a workgroup (arguments, counts, lists, first K/V tiles,
+ * dispatch) are paid once per workgroup instead of once per Q tile.
  *
- * sa_fwd_schedule_bytes   size of the schedule buffer for this problem on the CURRENT device (it depends on the
- *                         number of compute units); 0 when the forward has no persistent kernel for the tile
- *                         sizes (BQ must be 32, 64 or 128, BK a power of two >= 16 with Sk/BK <= 1024) or on
- *                         invalid arguments.
+ *   SA_SCHEDULE_PAIRS       one workgroup per two Q tiles of a pair of planes, tile r from the top with tile r
+ *                           from the bottom; the hardware dispatcher still balances the workgroups.
+ *   SA_SCHEDULE_PERSISTENT  two workgroups per compute unit of the CURRENT device; the Q tiles are dealt out in
+ *                           rounds by their cost (the list lengths), costliest tile to the least loaded workgroup.
+ *
+ * sa_fwd_schedule_bytes   size of the schedule buffer; 0 when the forward has no kernel for scheduled tiles at
+ *                         these sizes (BQ must be 32, 64 or 128, BK a power of two >= 16 with Sk/BK <= 1024), on
+ *                         invalid arguments, or (persistent mode) without a device.
  * sa_fwd_schedule         fills it from the two count tensors of sa_mask_classify (same stream, after it).  The
- *                         result depends on the counts, B, H, the tile sizes and the device only: compute it
- *                         once per mask and reuse it for every forward over that mask.
+ *                         result depends on the counts, B, H, the tile sizes, the mode and (persistent mode) the
+ *                         device only: compute it once per mask and reuse it for every forward over that mask.
  */
-size_t sa_fwd_schedule_bytes(int B, int H, int Sq, int Sk, int BQ, int BK);
+size_t sa_fwd_schedule_bytes(int B, int H, int Sq, int Sk, int BQ, int BK, int mode);
 int sa_fwd_schedule(const int32_t *full_lens, const int64_t full_lens_strides[3], const int32_t *part_lens,
-                    const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int BQ, int BK,
+                    const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int BQ, int BK, int mode,
                     int32_t *schedule, size_t schedule_bytes, void *stream);
 
 /*
@@ -171,9 +181,10 @@ int sa_fwd_schedule(const int32_t *full_lens, const int64_t full_lens_strides[3]
  *   packed, packed_strides   output of sa_mask_pack_partial for the same mask, tile sizes and lists (strides may
  *                            be 0 on broadcast dimensions), or NULL.  When given, `mask` is not read and may be
  *                            NULL, so the bool tensor can be released once the lists and the packed bits exist.
- *   schedule, schedule_bytes output of sa_fwd_schedule for the same counts and sizes on this device, or NULL
- *                            (then, and when schedule_bytes is not sa_fwd_schedule_bytes(...), one workgroup
- *                            per Q tile is launched as in sa_sparse_attention_fwd).
+ *   schedule, schedule_bytes, schedule_mode
+ *                            output of sa_fwd_schedule for the same counts, sizes and mode (on this device), or
+ *                            NULL (then, and when schedule_bytes is not sa_fwd_schedule_bytes(...), one
+ *                            workgroup per Q tile is launched as in sa_sparse_attention_fwd).
  */
 int sa_sparse_attention_fwd_ex(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
                                const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
@@ -182,9 +193,9 @@ int sa_sparse_attention_fwd_ex(const void *q, const int64_t q_strides[4], const 
                                const int64_t full_lens_strides[3], const int32_t *part_ids,
                                const int64_t part_ids_strides[4], const int32_t *part_lens,
                                const int64_t part_lens_strides[3], const uint8_t *packed,
-                               const int64_t packed_strides[2], const int32_t *schedule, size_t schedule_bytes, int B,
-                               int H, int Sq, int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2,
-                               void *stream);
+                               const int64_t packed_strides[2], const int32_t *schedule, size_t schedule_bytes,
+                               int schedule_mode, int B, int H, int Sq, int Sk, int D, int BQ, int BK, int dtype,
+                               float sm_scale_log2, void *stream);
 
 #ifdef __cplusplus
 }

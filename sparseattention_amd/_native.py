@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsparseattn_hip.so")
 
-SA_ABI_VERSION = 3
+SA_ABI_VERSION = 4
 SA_OK = 0
 SA_ERR_INVALID_ARGUMENT = -1
 SA_ERR_UNSUPPORTED = -2
@@ -19,6 +19,9 @@ SA_ERR_HIP = -4
 
 SA_DTYPE_BF16 = 0
 SA_DTYPE_FP16 = 1
+
+SA_SCHEDULE_PERSISTENT = 0
+SA_SCHEDULE_PAIRS = 1
 
 #: every symbol include/sparseattn.h declares
 EXPORTS = (
@@ -78,13 +81,13 @@ def load() -> ctypes.CDLL:
     lib.sa_mask_pack_partial.restype = ctypes.c_int
     lib.sa_mask_pack_partial.argtypes = [_vp, _i64p] + [ctypes.c_int] * 6 + [_vp, _i64p] * 3 + [_vp]
     lib.sa_fwd_schedule_bytes.restype = ctypes.c_size_t
-    lib.sa_fwd_schedule_bytes.argtypes = [ctypes.c_int] * 6
+    lib.sa_fwd_schedule_bytes.argtypes = [ctypes.c_int] * 7
     lib.sa_fwd_schedule.restype = ctypes.c_int
-    lib.sa_fwd_schedule.argtypes = [_vp, _i64p] * 2 + [ctypes.c_int] * 6 + [_vp, ctypes.c_size_t, _vp]
+    lib.sa_fwd_schedule.argtypes = [_vp, _i64p] * 2 + [ctypes.c_int] * 7 + [_vp, ctypes.c_size_t, _vp]
     lib.sa_sparse_attention_fwd_ex.restype = ctypes.c_int
     lib.sa_sparse_attention_fwd_ex.argtypes = (
         [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, ctypes.c_size_t]
-        + [ctypes.c_int] * 8 + [ctypes.c_float, _vp]
+        + [ctypes.c_int] * 9 + [ctypes.c_float, _vp]
     )
     if lib.sa_abi_version() != SA_ABI_VERSION:
         raise RuntimeError(f"libsparseattn_hip ABI {lib.sa_abi_version()} != expected {SA_ABI_VERSION}")

@@ -71,10 +71,49 @@ __global__ __launch_bounds__(64) void schedule_kernel(const ScheduleParams p) {
     if (is_wg) row[0] = int4{count, 0, 0, 0};
 }
 
+// Pairs: workgroup w takes two Q tiles of one pair of planes, the r-th costliest-first and the r-th from the other
+// end (under causal-like masks a long list with a short one, so that all workgroups carry the same load and
+// the hardware dispatcher still evens out what differs).  The last plane of an odd count pairs its own tiles.
+// One thread per schedule row g; rows are handed to XCDs in turn, so row g holds workgroup (g & 7) * G/8 + g / 8.
+__global__ __launch_bounds__(256) void schedule_pairs_kernel(const ScheduleParams p) {
+    const int g = blockIdx.x * 256 + threadIdx.x;
+    if (g >= p.G) return;
+    const int BH = p.B * p.H;
+    const int pairs = BH >> 1;
+    const int64_t w = (int64_t)(g & 7) * (p.G >> 3) + (g >> 3);
+    int4 *row = reinterpret_cast<int4 *>(p.sched) + (int64_t)g * (p.R + 1);
+    int bh[2], qt[2], n = 0;
+    if (w < (int64_t)pairs * p.nQ) {
+        const int pp = (int)(w / p.nQ), r = (int)(w - (int64_t)pp * p.nQ);
+        // position r of the pair's interleaved order: plane r & 1, tile nQ-1 - r/2; its mirror 2nQ-1-r
+        const int r2 = 2 * p.nQ - 1 - r;
+        bh[0] = 2 * pp + (r & 1), qt[0] = p.nQ - 1 - (r >> 1);
+        bh[1] = 2 * pp + (r2 & 1), qt[1] = p.nQ - 1 - (r2 >> 1);
+        n = 2;
+    } else if (BH & 1) {
+        const int64_t r = w - (int64_t)pairs * p.nQ;  // the unpaired plane: tile nQ-1-r with tile r
+        if (r < (p.nQ + 1) / 2) {
+            bh[0] = BH - 1, qt[0] = p.nQ - 1 - (int)r;
+            n = 1;
+            if ((int)r != p.nQ - 1 - (int)r) {
+                bh[1] = BH - 1, qt[1] = (int)r;
+                n = 2;
+            }
+        }
+    }
+    for (int i = 0; i < n; i++) {
+        const int b = bh[i] / p.H, h = bh[i] - b * p.H;
+        row[1 + i] = int4{(b << 16) | h, qt[i], p.full_lens[b * p.fls[0] + h * p.fls[1] + qt[i] * p.fls[2]],
+                          p.part_lens[b * p.pls[0] + h * p.pls[1] + qt[i] * p.pls[2]]};
+    }
+    row[0] = int4{n, 0, 0, 0};
+}
+
 }  // namespace
 
 hipError_t launch_schedule(const ScheduleParams &p, hipStream_t stream) {
-    hipLaunchKernelGGL(schedule_kernel, dim3(8), dim3(64), 0, stream, p);
+    if (p.pairs) hipLaunchKernelGGL(schedule_pairs_kernel, dim3((p.G + 255) / 256), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(schedule_kernel, dim3(8), dim3(64), 0, stream, p);
     return hipGetLastError();
 }
 

@@ -50,6 +50,7 @@ struct ScheduleParams {
     int B, H, nQ;
     int G, R;
     int lbk;  // log2(BK): chunks of 64 keys per entry = BK/64, entries per chunk = 64/BK
+    int pairs;  // 1: two Q tiles per workgroup, one workgroup per pair of tiles (G = number of pairs, R = 2)
     int32_t *sched;
 };
 

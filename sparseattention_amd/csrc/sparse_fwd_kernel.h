@@ -450,6 +450,40 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         }
     };
 
+    // The mask of 32-key block KB of a chunk, applied to its scores: entries the mask leaves out become -inf.
+    // Bit j of `valid` / `part`: list entry j of the chunk exists / is PARTIAL.
+    auto apply_mask_block = [&](f32x16 &sb, auto kb_c, unsigned valid, unsigned part, const uint32_t(&mk)[NMW]) {
+        constexpr int kb = decltype(kb_c)::value;
+        if constexpr (PK) {
+            // bit k of w: key k of this 32-key block; FULL entries count as all ones, absent ones as zero
+            auto word = [&](int j, uint32_t ones) -> uint32_t {
+                return ((part >> j) & 1u) ? mk[j] : (((valid >> j) & 1u) ? ones : 0u);
+            };
+            uint32_t w;
+            if constexpr (MODE == 0) w = word(2 * kb, 0xffffu) | (word(2 * kb + 1, 0xffffu) << 16);
+            else if constexpr (MODE == 1) w = word(kb, ~0u);
+            else w = (valid & 1u) ? mk[kb] : 0u;  // a chunk of a PARTIAL entry (or of an absent one)
+            w >>= sh4;  // this lane's keys are 8g + 4hh + jj
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) {
+                    const uint32_t keep = (uint32_t)__builtin_amdgcn_sbfe((int)w, 8 * g + jj, 1);  // 0 or ~0
+                    const uint32_t x = __float_as_uint(sb[4 * g + jj]);
+                    sb[4 * g + jj] = __uint_as_float((x & keep) | (0xff800000u & ~keep));
+                }
+        } else {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int j = MODE == 0 ? 2 * kb + (g >> 1) : (MODE == 1 ? kb : 0);  // list entry of this group
+                const uint32_t w = ((valid >> j) & 1u) ? mk[4 * kb + g] : 0u;
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++)
+                    if (((w >> (8 * jj)) & 0xffu) == 0u) sb[4 * g + jj] = kNegInf;
+            }
+        }
+    };
+
     // One chunk from stage BUF, in two phases.
     // S phase: s = K . Q^T - m_ref.  When `fetch`, the pieces of the chunk planned in `pl` are sent to stage
     // FBUF between its MFMA bundles.
@@ -489,39 +523,8 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         constexpr int BUF = decltype(buf_c)::value;
         const uint8_t *vb_ = smem + NS * KBUF + BUF * VBUF;
         if (special) {
-            if constexpr (PK) {
-#pragma unroll
-                for (int kb = 0; kb < 2; kb++) {
-                    // bit k of w: key k of this 32-key block; FULL entries count as all ones, absent ones as zero
-                    auto word = [&](int j, uint32_t ones) -> uint32_t {
-                        return ((part >> j) & 1u) ? mk[j] : (((valid >> j) & 1u) ? ones : 0u);
-                    };
-                    uint32_t w;
-                    if constexpr (MODE == 0) w = word(2 * kb, 0xffffu) | (word(2 * kb + 1, 0xffffu) << 16);
-                    else if constexpr (MODE == 1) w = word(kb, ~0u);
-                    else w = (valid & 1u) ? mk[kb] : 0u;  // a chunk of a PARTIAL entry (or of an absent one)
-                    w >>= sh4;  // this lane's keys are 8g + 4hh + jj
-#pragma unroll
-                    for (int g = 0; g < 4; g++)
-#pragma unroll
-                        for (int jj = 0; jj < 4; jj++) {
-                            const uint32_t keep = (uint32_t)__builtin_amdgcn_sbfe((int)w, 8 * g + jj, 1);  // 0 or ~0
-                            const uint32_t x = __float_as_uint(s[kb][4 * g + jj]);
-                            s[kb][4 * g + jj] = __uint_as_float((x & keep) | (0xff800000u & ~keep));
-                        }
-                }
-            } else {
-#pragma unroll
-                for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        const int j = MODE == 0 ? 2 * kb + (g >> 1) : (MODE == 1 ? kb : 0);  // list entry of this group
-                        const uint32_t w = ((valid >> j) & 1u) ? mk[4 * kb + g] : 0u;
-#pragma unroll
-                        for (int jj = 0; jj < 4; jj++)
-                            if (((w >> (8 * jj)) & 0xffu) == 0u) s[kb][4 * g + jj] = kNegInf;
-                    }
-            }
+            apply_mask_block(s[0], std::integral_constant<int, 0>{}, valid, part, mk);
+            apply_mask_block(s[1], std::integral_constant<int, 1>{}, valid, part, mk);
         }
 
         // Online softmax in exp2 units (sparse_attn_kernel.py:47-58), with a lagging reference value: s holds

@@ -141,10 +141,23 @@ namespace {
 // Workgroups the persistent forward launches on the current device (2 per compute unit, a multiple of 8, at
 // most 512), entries per schedule row, and the bytes of the schedule; 0 when there is no persistent kernel for
 // the problem or no device.
-size_t schedule_shape(int B, int H, int Sq, int Sk, int BQ, int BK, int *G_out, int *R_out) {
+size_t schedule_shape(int B, int H, int Sq, int Sk, int BQ, int BK, int mode, int *G_out, int *R_out) {
     if (B <= 0 || H <= 0 || Sq <= 0 || Sk <= 0 || BQ <= 0 || BK <= 0 || Sq % BQ || Sk % BK) return 0;
     if (BQ != 32 && BQ != 64 && BQ != 128) return 0;
     if (log2_exact(BK) < 4 || Sk / BK > 1024 || B >= 32768 || H >= 65536) return 0;
+    if (mode == SA_SCHEDULE_PAIRS) {
+        // one workgroup per two Q tiles (per one for the middle tile of an unpaired plane), rounded up to whole
+        // groups of 8 rows
+        const int nQ = Sq / BQ;
+        const int64_t BH = (int64_t)B * H;
+        int64_t W = (BH / 2) * nQ + ((BH & 1) ? (nQ + 1) / 2 : 0);
+        W = (W + 7) / 8 * 8;
+        if (W > 0x7fffffffLL) return 0;
+        if (G_out) *G_out = (int)W;
+        if (R_out) *R_out = 2;
+        return (size_t)W * 3 * 16;
+    }
+    if (mode != SA_SCHEDULE_PERSISTENT) return 0;
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess) return 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
@@ -167,8 +180,8 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
                  const int32_t *full_lens, const int64_t full_lens_strides[3], const int32_t *part_ids,
                  const int64_t part_ids_strides[4], const int32_t *part_lens, const int64_t part_lens_strides[3],
                  const uint8_t *packed, const int64_t packed_strides[2], bool use_packed, const int32_t *schedule,
-                 size_t schedule_bytes, int B, int H, int Sq, int Sk, int D, int BQ, int BK, int dtype,
-                 float sm_scale_log2, void *stream) {
+                 size_t schedule_bytes, int schedule_mode, int B, int H, int Sq, int Sk, int D, int BQ, int BK,
+                 int dtype, float sm_scale_log2, void *stream) {
     g_error[0] = 0;
     if (!q || !k || !v || !o || !q_strides || !k_strides || !v_strides || !o_strides || !full_ids ||
         !full_ids_strides || !full_lens || !full_lens_strides || !part_ids || !part_ids_strides || !part_lens ||
@@ -232,7 +245,7 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
     fp.sched = nullptr;
     if (schedule) {
         int G = 0, R = 0;
-        const size_t want = schedule_shape(B, H, Sq, Sk, BQ, BK, &G, &R);
+        const size_t want = schedule_shape(B, H, Sq, Sk, BQ, BK, schedule_mode, &G, &R);
         if (want != 0 && want == schedule_bytes) {
             if (!aligned(schedule, 16))
                 return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd_ex: schedule needs a 16-byte aligned base");
@@ -286,7 +299,7 @@ int sa_sparse_attention_fwd(const void *q, const int64_t q_strides[4], const voi
                             int dtype, float sm_scale_log2, void *stream) {
     return forward_impl(q, q_strides, k, k_strides, v, v_strides, o, o_strides, mask, mask_strides, full_ids,
                         full_ids_strides, full_lens, full_lens_strides, part_ids, part_ids_strides, part_lens,
-                        part_lens_strides, nullptr, nullptr, false, nullptr, 0, B, H, Sq, Sk, D, BQ, BK, dtype,
+                        part_lens_strides, nullptr, nullptr, false, nullptr, 0, 0, B, H, Sq, Sk, D, BQ, BK, dtype,
                         sm_scale_log2, stream);
 }
 
@@ -297,9 +310,9 @@ int sa_sparse_attention_fwd_ex(const void *q, const int64_t q_strides[4], const 
                                const int64_t full_lens_strides[3], const int32_t *part_ids,
                                const int64_t part_ids_strides[4], const int32_t *part_lens,
                                const int64_t part_lens_strides[3], const uint8_t *packed,
-                               const int64_t packed_strides[2], const int32_t *schedule, size_t schedule_bytes, int B,
-                               int H, int Sq, int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2,
-                               void *stream) {
+                               const int64_t packed_strides[2], const int32_t *schedule, size_t schedule_bytes,
+                               int schedule_mode, int B, int H, int Sq, int Sk, int D, int BQ, int BK, int dtype,
+                               float sm_scale_log2, void *stream) {
     const bool use_packed = packed != nullptr;
     if (use_packed) {
         g_error[0] = 0;
@@ -309,25 +322,27 @@ int sa_sparse_attention_fwd_ex(const void *q, const int64_t q_strides[4], const 
     }
     return forward_impl(q, q_strides, k, k_strides, v, v_strides, o, o_strides, mask, mask_strides, full_ids,
                         full_ids_strides, full_lens, full_lens_strides, part_ids, part_ids_strides, part_lens,
-                        part_lens_strides, packed, packed_strides, use_packed, schedule, schedule_bytes, B, H, Sq, Sk,
-                        D, BQ, BK, dtype, sm_scale_log2, stream);
+                        part_lens_strides, packed, packed_strides, use_packed, schedule, schedule_bytes, schedule_mode,
+                        B, H, Sq, Sk, D, BQ, BK, dtype, sm_scale_log2, stream);
 }
 
-size_t sa_fwd_schedule_bytes(int B, int H, int Sq, int Sk, int BQ, int BK) {
-    return schedule_shape(B, H, Sq, Sk, BQ, BK, nullptr, nullptr);
+size_t sa_fwd_schedule_bytes(int B, int H, int Sq, int Sk, int BQ, int BK, int mode) {
+    return schedule_shape(B, H, Sq, Sk, BQ, BK, mode, nullptr, nullptr);
 }
 
 int sa_fwd_schedule(const int32_t *full_lens, const int64_t full_lens_strides[3], const int32_t *part_lens,
-                    const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int BQ, int BK,
+                    const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int BQ, int BK, int mode,
                     int32_t *schedule, size_t schedule_bytes, void *stream) {
     g_error[0] = 0;
     if (!full_lens || !full_lens_strides || !part_lens || !part_lens_strides || !schedule)
         return fail(SA_ERR_INVALID_ARGUMENT, "sa_fwd_schedule: null pointer argument");
     if (const int rc = check_tiling(B, H, Sq, Sk, BQ, BK)) return rc;
     int G = 0, R = 0;
-    const size_t want = schedule_shape(B, H, Sq, Sk, BQ, BK, &G, &R);
+    if (mode != SA_SCHEDULE_PERSISTENT && mode != SA_SCHEDULE_PAIRS)
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_fwd_schedule: mode %d (0 = persistent, 1 = pairs)", mode);
+    const size_t want = schedule_shape(B, H, Sq, Sk, BQ, BK, mode, &G, &R);
     if (want == 0)
-        return fail(SA_ERR_UNSUPPORTED, "sa_fwd_schedule: no persistent forward for BLOCK_Q %d, BLOCK_K %d, Sk %d (BLOCK_Q 32/64/128, BLOCK_K a power of two >= 16, Sk/BLOCK_K <= 1024), or no device", BQ, BK, Sk);
+        return fail(SA_ERR_UNSUPPORTED, "sa_fwd_schedule: no scheduled forward for BLOCK_Q %d, BLOCK_K %d, Sk %d (BLOCK_Q 32/64/128, BLOCK_K a power of two >= 16, Sk/BLOCK_K <= 1024), or no device", BQ, BK, Sk);
     if (schedule_bytes != want)
         return fail(SA_ERR_WORKSPACE, "sa_fwd_schedule: schedule of %zu bytes required, %zu given", want, schedule_bytes);
     if (!aligned(schedule, 16)) return fail(SA_ERR_UNSUPPORTED, "sa_fwd_schedule: schedule needs a 16-byte aligned base");
@@ -344,6 +359,7 @@ int sa_fwd_schedule(const int32_t *full_lens, const int64_t full_lens_strides[3]
     sp.G = G;
     sp.R = R;
     sp.lbk = log2_exact(BK);
+    sp.pairs = mode == SA_SCHEDULE_PAIRS ? 1 : 0;
     sp.sched = schedule;
     const hipError_t e = sa::launch_schedule(sp, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_fwd_schedule: launch failed: %s", hipGetErrorString(e));

@@ -28,10 +28,11 @@ class MaskMetadata:
     ``masked_kv_ids[b,h,qt,slot]``: rows first, entry (r, c) in bit ``c & 7`` of byte ``(r*BK + c) >> 3``.
     When present, :func:`sparse_attention` reads these bits and never touches the bool mask.
 
-    ``schedule`` is the second addition (optional, default None): int32 [workgroups, rounds + 1, 4], which Q tiles
-    each of the forward's persistent workgroups processes, in order (entry 0 of a row: the count; then
-    ``((b << 16) | h, qt, unmasked_len, masked_len)`` per tile).  It depends on the counts, on B and H and on
-    the device; without it the forward launches one workgroup per Q tile.
+    ``schedule`` / ``schedule_mode`` are the second addition (optional, default None): int32
+    [workgroups, rounds + 1, 4], which Q tiles each workgroup of the forward processes, in order (entry 0 of a
+    row: the count; then ``((b << 16) | h, qt, unmasked_len, masked_len)`` per tile), made by
+    ``compute_mask_kernel(..., schedule="pairs" | "persistent")``.  It depends on the counts, on B and H and, for
+    "persistent", on the device; without it the forward launches one workgroup per Q tile.
     """
 
     unmasked_kv_ids: torch.Tensor
@@ -40,6 +41,7 @@ class MaskMetadata:
     masked_lens: torch.Tensor
     packed_masks: Optional[torch.Tensor] = None
     schedule: Optional[torch.Tensor] = None
+    schedule_mode: int = 0
 
 
 def _check_mask(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int):
@@ -82,7 +84,7 @@ def compute_mask_slow(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int) -> MaskMet
 
 
 def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int, pack_partial: Optional[bool] = None,
-                        schedule: bool = False) -> MaskMetadata:
+                        schedule=None) -> MaskMetadata:
     """Classify the mask's tiles on the GPU (replaces mask_utils.py:85-107).
 
     ``mask``: bool [B,H,Sq,Sk] on a ROCm device, any strides.  Dimensions that are broadcast in
@@ -92,10 +94,13 @@ def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int, pack_par
 
     ``pack_partial``: also fill ``MaskMetadata.packed_masks`` (Sq*Sk/8 bytes per distinct mask plane).
     Default: whenever BLOCK_K is a multiple of 8; ``False`` gives exactly the reference's four tensors.
-    ``schedule``: also fill ``MaskMetadata.schedule`` (needs BLOCK_Q 32/64/128, BLOCK_K a power of two >= 16
-    and at most 1024 KV tiles per row).  Off by default: measured on MI355X, persistent workgroups win when the
-    lists are short (a few hundred keys per Q tile) and lose a few percent to the hardware dispatcher when
-    they are long, because a static hand-out cannot follow the uneven pace of the workgroups that share a CU.
+    ``schedule``: ``"pairs"`` or ``"persistent"`` also fills ``MaskMetadata.schedule`` (needs BLOCK_Q 32/64/128,
+    BLOCK_K a power of two >= 16 and at most 1024 KV tiles per row); ``None``/``False`` leaves it out.
+    "pairs": one workgroup per two Q tiles, tile r from the top with tile r from the bottom of a pair of planes.
+    "persistent": as many workgroups as the device holds, each with a list of Q tiles ranked by cost; measured
+    on MI355X it wins when the lists are short (a few hundred keys per Q tile) and loses a few percent to the
+    hardware dispatcher when they are long, because a static hand-out cannot follow the uneven pace of the
+    workgroups that share a compute unit.
     """
     B, H, Sq, Sk = _check_mask(mask, BLOCK_Q, BLOCK_K)
     if not mask.is_cuda:
@@ -141,19 +146,27 @@ def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int, pack_par
             _native.check(rc)
             packed = packed.expand(B, H, nQ, nK, BLOCK_Q * BLOCK_K // 8)
         sched = None
+        mode = 0
         if schedule:
-            nbytes = int(lib.sa_fwd_schedule_bytes(B, H, Sq, Sk, BLOCK_Q, BLOCK_K))
+            modes = {"persistent": _native.SA_SCHEDULE_PERSISTENT, "pairs": _native.SA_SCHEDULE_PAIRS,
+                     True: _native.SA_SCHEDULE_PAIRS}
+            if schedule not in modes:
+                raise ValueError(f"schedule must be 'pairs', 'persistent' or None (got {schedule!r})")
+            mode = modes[schedule]
+            nbytes = int(lib.sa_fwd_schedule_bytes(B, H, Sq, Sk, BLOCK_Q, BLOCK_K, mode))
             if nbytes == 0:
-                raise ValueError(f"no persistent forward for BLOCK_Q={BLOCK_Q}, BLOCK_K={BLOCK_K}, Sk={Sk}")
-            if nbytes:
-                sched = torch.empty(nbytes // 4, dtype=torch.int32, device=dev)
-                rc = lib.sa_fwd_schedule(fl.data_ptr(), _native.strides(fl.stride()), pl.data_ptr(),
-                                         _native.strides(pl.stride()), B, H, Sq, Sk, BLOCK_Q, BLOCK_K,
-                                         sched.data_ptr(), nbytes, torch.cuda.current_stream(dev).cuda_stream)
-                _native.check(rc)
+                raise ValueError(f"no scheduled forward for BLOCK_Q={BLOCK_Q}, BLOCK_K={BLOCK_K}, Sk={Sk}")
+            sched = torch.empty(nbytes // 4, dtype=torch.int32, device=dev)
+            rc = lib.sa_fwd_schedule(fl.data_ptr(), _native.strides(fl.stride()), pl.data_ptr(),
+                                     _native.strides(pl.stride()), B, H, Sq, Sk, BLOCK_Q, BLOCK_K, mode,
+                                     sched.data_ptr(), nbytes, torch.cuda.current_stream(dev).cuda_stream)
+            _native.check(rc)
+            if mode == _native.SA_SCHEDULE_PAIRS:
+                sched = sched.view(-1, 3, 4)
+            else:
                 G = min(2 * torch.cuda.get_device_properties(dev).multi_processor_count, 512) & ~7
                 sched = sched.view(G, nbytes // (16 * G), 4)
-    return MaskMetadata(fid, fl, pid, pl, packed, sched)
+    return MaskMetadata(fid, fl, pid, pl, packed, sched, mode)
 
 
 # Tile sizes tried by select_block_sizes, and what one executed mask entry costs at each BLOCK_Q relative to

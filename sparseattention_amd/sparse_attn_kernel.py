@@ -79,7 +79,8 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
         sched = getattr(mask_metadata, "schedule", None)
         if packed is not None or sched is not None:
             pk = (packed.data_ptr(), S(packed.stride()[:2])) if packed is not None else (None, None)
-            sc = (sched.data_ptr(), sched.numel() * 4) if sched is not None else (None, 0)
+            sc = ((sched.data_ptr(), sched.numel() * 4, int(getattr(mask_metadata, "schedule_mode", 0)))
+                  if sched is not None else (None, 0, 0))
             rc = lib.sa_sparse_attention_fwd_ex(*common, *pk, *sc, *tail)
         else:
             rc = lib.sa_sparse_attention_fwd(*common, *tail)

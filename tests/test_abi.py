@@ -128,8 +128,8 @@ def test_extended_forward_rejects_bad_arguments():
 
     def call(packed=FAKE, ps=_native.strides((0, 0)), mask=None, BK=32, B=1, sched=None, sched_bytes=0):
         return lib.sa_sparse_attention_fwd_ex(FAKE, qs, FAKE, qs, FAKE, qs, FAKE, qs, mask, None, FAKE, I4, FAKE, S3,
-                                              FAKE, I4, FAKE, S3, packed, ps, sched, sched_bytes, B, 1, 256, 256, 128,
-                                              128, BK, 0, 0.1, None)
+                                              FAKE, I4, FAKE, S3, packed, ps, sched, sched_bytes, 0, B, 1, 256, 256,
+                                              128, 128, BK, 0, 0.1, None)
 
     # neither a mask nor packed bits
     assert call(packed=None) == _native.SA_ERR_INVALID_ARGUMENT and "mask" in last_error()
@@ -145,19 +145,25 @@ def test_extended_forward_rejects_bad_arguments():
 def test_schedule_rejects_bad_arguments():
     lib = _native.load()
 
-    def call(fl=FAKE, sched=FAKE, nbytes=16, Sq=256, BQ=128, BK=32):
-        return lib.sa_fwd_schedule(fl, S3, FAKE, S3, 1, 1, Sq, 256, BQ, BK, sched, nbytes, None)
+    def call(fl=FAKE, sched=FAKE, nbytes=16, Sq=256, BQ=128, BK=32, mode=0):
+        return lib.sa_fwd_schedule(fl, S3, FAKE, S3, 1, 1, Sq, 256, BQ, BK, mode, sched, nbytes, None)
 
     assert call(fl=None) == _native.SA_ERR_INVALID_ARGUMENT and "null" in last_error()
     assert call(sched=None) == _native.SA_ERR_INVALID_ARGUMENT
     assert call(Sq=200) == _native.SA_ERR_INVALID_ARGUMENT
     # tile sizes without a persistent kernel (and, without a GPU, every size): unsupported, nothing launched
-    assert call(BQ=256) == _native.SA_ERR_UNSUPPORTED and "persistent" in last_error()
+    assert call(BQ=256) == _native.SA_ERR_UNSUPPORTED and "scheduled" in last_error()
     assert call(BK=8) == _native.SA_ERR_UNSUPPORTED
-    assert lib.sa_fwd_schedule_bytes(1, 1, 256, 256, 256, 32) == 0
-    assert lib.sa_fwd_schedule_bytes(1, 1, 256, 256, 100, 32) == 0
+    assert call(mode=7) == _native.SA_ERR_INVALID_ARGUMENT
+    assert lib.sa_fwd_schedule_bytes(1, 1, 256, 256, 256, 32, 0) == 0
+    assert lib.sa_fwd_schedule_bytes(1, 1, 256, 256, 100, 32, 1) == 0
+    # pairs: one row of three entries per two Q tiles, in whole groups of 8 rows; no device needed for the size
+    assert lib.sa_fwd_schedule_bytes(8, 32, 4096, 4096, 128, 32, 1) == 4096 * 3 * 16
+    assert lib.sa_fwd_schedule_bytes(1, 1, 256, 256, 128, 32, 1) == 8 * 3 * 16
+    assert lib.sa_fwd_schedule_bytes(1, 3, 384, 256, 128, 32, 1) == 8 * 3 * 16    # 3 + 2 workgroups -> 8 rows
+    assert call(mode=1, nbytes=16) == _native.SA_ERR_WORKSPACE
     if not torch.cuda.is_available():
-        assert lib.sa_fwd_schedule_bytes(1, 1, 256, 256, 128, 32) == 0
+        assert lib.sa_fwd_schedule_bytes(1, 1, 256, 256, 128, 32, 0) == 0
         assert call() == _native.SA_ERR_UNSUPPORTED
 
 
