@@ -919,10 +919,12 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
                 constexpr int cur = j & 1, nxt = cur ^ 1;
                 const int tc = t + j;
                 if (tc < T) {
-                    const bool fetch = tc + 1 < T;
                     if (sp[nxt]) load_mask(tc + 1, coln, mk[nxt], MaskSrc{mrow, prow, F, NE});
                     f32x16 s[2];
-                    phase_s(jc, s, std::integral_constant<int, nxt>{}, fetch, pl);
+                    // the fetch is unconditional: after the last chunk the plan is the clamped one and the last
+                    // chunk is fetched once more, into the stage nobody reads any more (cheaper than a branch in
+                    // front of every direct load)
+                    phase_s(jc, s, std::integral_constant<int, nxt>{}, true, pl);
                     const int t2 = tc + 2 < T ? tc + 2 : T - 1, t3 = tc + 3 < T ? tc + 3 : T - 1;
                     int col2[EPC];
                     unsigned valid2 = 0u, part2 = 0u;
