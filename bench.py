@@ -3,10 +3,11 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-sweep] [--no-cpu]
 
-A step is one forward pass (sa_sparse_attention_fwd) over the headline workload: causal bool mask
-passed as a tensor, B=8 H=32 S=4096 D=128 bf16, tiles 128x32, inputs and the precomputed tile lists
-resident in HBM (the reference also excludes preprocessing from the forward time and reports it
-separately, test_attn.py:38,65,68).  Prints ONE JSON line.
+A step is one forward pass (sa_sparse_attention_fwd_ex) over the headline workload: causal bool mask
+passed as a tensor, B=8 H=32 S=4096 D=128 bf16, tiles 128x32, inputs and the precomputed mask metadata
+(tile lists, bit-packed partial tiles, pairs schedule: what compute_mask_kernel returns) resident in HBM;
+the reference also excludes preprocessing from the forward time and reports it separately
+(test_attn.py:38,65,68).  Prints ONE JSON line.
 
   value      effective TFLOP/s by the reference's convention: 4*B*H*Sq*Sk*D * mean(mask) / time
              (test_attn.py:84, :108-111)
@@ -14,6 +15,8 @@ separately, test_attn.py:38,65,68).  Prints ONE JSON line.
              (full + partial tiles) * 4*BQ*BK*D flop per launch / mean launch duration (HIP events)
   mask_classify   the preprocessing kernels on a 1 GiB mask against the HBM peak
   across_p   the same forward on random block masks of sparsity p, a dense mask and the causal one
+  variants   the headline workload through the other routes of the library (bool-mask reads, no schedule,
+             persistent workgroups)
   cpu_baseline / cpu_sdpa_baseline   the CPU oracle and torch's masked SDPA on a bounded sample
 """
 import argparse
@@ -32,8 +35,8 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E peak, GB/s
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this script and scaled by
 # the readings of a 1 GiB device copy in the same run (--calibrate-copy).  The summaries with the commands
 # are profiles/sparse_fwd_kernel_causal_B8H32S4096D128.txt and profiles/mask_classify_kernels_mask_32768x32768.txt.
-TRAFFIC_FWD_CAUSAL_BYTES = 1.3256e9      # 1007.6 MiB read + 256.6 MiB written
-TRAFFIC_CLASSIFY_1GIB_BYTES = 1.0745e9   # 1,048,648 + 331 KiB read, 256 + 45.5 KiB written
+TRAFFIC_FWD_CAUSAL_BYTES = 1.3566e9      # 1037.8 MiB read + 256.0 MiB written
+TRAFFIC_CLASSIFY_1GIB_BYTES = 1.0744e9   # 1,048,622 + 327 KiB read, 256 + 45.5 KiB written
 
 B, H, S, D = 8, 32, 4096, 128
 BQ, BK = 128, 32
@@ -75,12 +78,12 @@ def time_launches(fn, steps, warmup):
     return wall_ms, ev_ms
 
 
-def forward_case(name, mask2d, q, k, v, steps, warmup):
+def forward_case(name, mask2d, q, k, v, steps, warmup, schedule=None, pack_partial=None):
     import torch
     from sparseattention_amd import compute_mask_kernel, sparse_attention
 
     me = mask2d[None, None].expand(B, H, S, S)
-    md = compute_mask_kernel(me, BQ, BK)
+    md = compute_mask_kernel(me, BQ, BK, pack_partial=pack_partial, schedule=schedule)
     tiles_plane = int(md.unmasked_lens[0, 0].sum()) + int(md.masked_lens[0, 0].sum())
     partial_plane = int(md.masked_lens[0, 0].sum())
     frac = float(mask2d.float().mean())
@@ -127,10 +130,20 @@ def classify_case(steps, warmup):
         _native.check(rc)
 
     wall_ms, ev_ms = time_launches(run, steps, warmup)
+    # the optional extra step: one bit per entry of the PARTIAL tiles (1920 of 262144 tiles here)
+    packed = torch.empty(lib.sa_mask_pack_partial_bytes(ms, 1, 1, Sbig, Sbig, BQ, BK), dtype=torch.uint8, device="cuda")
+
+    def run_pack():
+        rc = lib.sa_mask_pack_partial(mask.data_ptr(), ms, 1, 1, Sbig, Sbig, BQ, BK, pid.data_ptr(), st(pid.stride()),
+                                      pl.data_ptr(), st(pl.stride()), packed.data_ptr(), st((0, 0)), stream)
+        _native.check(rc)
+
+    _, pack_ms = time_launches(run_pack, steps, warmup)
     nbytes = Sbig * Sbig + nQ * (2 * nK + 2) * 4  # mask read once + lists and counts written
     return {
         "workload": "sa_mask_classify on the composed mask, bool [32768,32768] = 1 GiB, tiles 128x32",
         "ms": round(ev_ms, 4),
+        "pack_partial_ms": round(pack_ms, 4),
         "roofline": {"bound": "hbm", "achieved": round(nbytes / (ev_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(nbytes / (ev_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                      "traffic": TRAFFIC_CLASSIFY_1GIB_BYTES, "algorithmic_bytes": nbytes},
@@ -143,8 +156,10 @@ def classify_small_case(steps, warmup):
     from sparseattention_amd import compute_mask_kernel, workloads as W
 
     me = W.causal_mask(S, "cuda")[None, None].expand(B, H, S, S)
-    wall_ms, ev_ms = time_launches(lambda: compute_mask_kernel(me, BQ, BK), steps, warmup)
-    return {"workload": "compute_mask_kernel on the causal mask [4096,4096] = 16 MiB (latency bound)", "ms": round(ev_ms, 4)}
+    wall_ms, ev_ms = time_launches(lambda: compute_mask_kernel(me, BQ, BK, pack_partial=False), steps, warmup)
+    _, full_ms = time_launches(lambda: compute_mask_kernel(me, BQ, BK, schedule="pairs"), steps, warmup)
+    return {"workload": "compute_mask_kernel on the causal mask [4096,4096] = 16 MiB (latency bound)",
+            "ms": round(ev_ms, 4), "with_pack_and_schedule_ms": round(full_ms, 4)}
 
 
 def cpu_baselines():
@@ -214,7 +229,7 @@ def main():
     torch.cuda.set_device(0)
     q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=0, device="cuda")
 
-    head = forward_case("causal", W.causal_mask(S, "cuda"), q, k, v, args.steps, args.warmup)
+    head = forward_case("causal", W.causal_mask(S, "cuda"), q, k, v, args.steps, args.warmup, schedule="pairs")
     achieved = head["_executed_flop"] / (head["kernel_ms"] * 1e-3) / 1e12
     result = {
         "metric": "effective TFLOP/s of the block-sparse forward (4*B*H*S*S*D*mean(mask)/time), B8 H32 S4096 D128 bf16",
@@ -230,7 +245,8 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "configs[1]: causal bool mask [4096,4096] passed as a tensor, B=8 H=32 S=4096 D=128 bf16, "
-                               "q/k/v ~ N(0,1), tiles BLOCK_Q=128 BLOCK_K=32, tile lists precomputed",
+                               "q/k/v ~ N(0,1), tiles BLOCK_Q=128 BLOCK_K=32, mask metadata precomputed "
+                               "(tile lists, bit-packed partial tiles, pairs schedule)",
                    "executed_tiles_per_plane": int(head["_executed_flop"] // (B * H * FLOP_PER_TILE)),
                    "partial_tiles_per_plane": head["partial_tiles_per_plane"]},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
@@ -239,6 +255,14 @@ def main():
                      "flop_per_launch": head["_executed_flop"]},
     }
     if not args.no_sweep:
+        vs, vw = max(5, args.steps // 2), max(2, args.warmup // 2)
+        causal = W.causal_mask(S, "cuda")
+        result["variants"] = {
+            name: round(forward_case(name, causal, q, k, v, vs, vw, schedule=sch, pack_partial=pk)["kernel_ms"], 4)
+            for name, sch, pk in (("pairs_schedule_packed_ms", "pairs", True), ("no_schedule_packed_ms", None, True),
+                                  ("no_schedule_bool_mask_ms", None, False),
+                                  ("persistent_schedule_packed_ms", "persistent", True))}
+        del causal
         rows = [head]
         sweep_steps, sweep_warm = max(5, args.steps // 5), max(2, args.warmup // 3)
         rows.append(forward_case("dense (all True)", torch.ones(S, S, dtype=torch.bool, device="cuda"), q, k, v,
