@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define SA_ABI_VERSION 4
+#define SA_ABI_VERSION 5
 
 enum sa_status {
     SA_OK = 0,
@@ -196,6 +196,34 @@ int sa_sparse_attention_fwd_ex(const void *q, const int64_t q_strides[4], const 
                                const int64_t packed_strides[2], const int32_t *schedule, size_t schedule_bytes,
                                int schedule_mode, int B, int H, int Sq, int Sk, int D, int BQ, int BK, int dtype,
                                float sm_scale_log2, void *stream);
+
+/*
+ * The forward for few query rows against a long K/V (decode): Sq <= 32 rows form the single Q tile of every (b, h),
+ * BLOCK_Q = Sq.  The result is that of sparse_attention (sparseattention/sparse_attn_kernel.py:149-185) called with
+ * BLOCK_Q = Sq; the reference has no kernel of its own for this shape ("Backwards pass + decode kernels" is item 3
+ * of its README's list of what could come next, README.md:65), and its one-program-per-Q-tile launch
+ * (sparse_attn_kernel.py:166) would leave one program per (b, h).  Here the list of every (b, h) is cut into
+ * num_splits ranges of 32-key chunks, one workgroup each, and a second kernel merges the partial results.
+ *
+ *   lists        output of sa_mask_classify for the same mask with BQ = Sq: shapes [B,H,1,Sk/BK] and [B,H,1]
+ *                (stride entry 2 is ignored)
+ *   BK           power of two >= 32
+ *   num_splits   workgroups per (b, h), 1..256, or 0 for sa_decode_num_splits(...)
+ *   workspace    sa_decode_workspace_bytes(...) bytes of device memory, 16-byte aligned (may be NULL when that is 0,
+ *                i.e. for one split); contents on return are unspecified
+ * q, k, v, o, D, dtype, sm_scale_log2, stream: as for sa_sparse_attention_fwd.
+ */
+int sa_decode_num_splits(int B, int H, int Sq, int Sk, int BK);
+size_t sa_decode_workspace_bytes(int B, int H, int Sq, int D, int num_splits);
+int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                               const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
+                               const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
+                               const int64_t full_ids_strides[4], const int32_t *full_lens,
+                               const int64_t full_lens_strides[3], const int32_t *part_ids,
+                               const int64_t part_ids_strides[4], const int32_t *part_lens,
+                               const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int D, int BK,
+                               int dtype, float sm_scale_log2, int num_splits, void *workspace, size_t workspace_bytes,
+                               void *stream);
 
 #ifdef __cplusplus
 }

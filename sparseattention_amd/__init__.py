@@ -3,6 +3,8 @@
 Same Python surface as tomatillos/sparseattention for its one hot path:
 
 * :func:`sparse_attention` (reference: ``sparseattention/sparse_attn_kernel.py:149``)
+* :func:`sparse_attention_decode`: the same function for Sq <= 32 with a split-KV launch (the reference names
+  decode kernels as future work, ``README.md:65``)
 * :func:`compute_mask_kernel`, :func:`compute_mask_slow`, :class:`MaskMetadata`
   (reference: ``sparseattention/mask_utils.py:85``, ``:14``, ``:6``)
 
@@ -10,6 +12,7 @@ The device work is done by hand-written gfx950 HIP kernels in ``libsparseattn_hi
 behind the C ABI of ``include/sparseattn.h``.
 """
 from .mask_utils import MaskMetadata, compute_mask_kernel, compute_mask_slow, select_block_sizes
-from .sparse_attn_kernel import sparse_attention
+from .sparse_attn_kernel import sparse_attention, sparse_attention_decode
 
-__all__ = ["MaskMetadata", "compute_mask_kernel", "compute_mask_slow", "select_block_sizes", "sparse_attention"]
+__all__ = ["MaskMetadata", "compute_mask_kernel", "compute_mask_slow", "select_block_sizes", "sparse_attention",
+           "sparse_attention_decode"]

@@ -135,5 +135,13 @@ constexpr int kListCap = 2048;
 // Persistent workgroups keep two lists in the same space, of the Q tile at hand and of the next one.
 constexpr int kPsListCap = 1024;
 
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {  // f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
+
 }  // namespace
 }  // namespace sa

@@ -84,4 +84,23 @@ struct FwdParams {
 // dtype: 0 bf16, 1 fp16.  Returns hipErrorInvalidValue when no instantiation matches (D, BQ).
 hipError_t launch_fwd(const FwdParams &p, int dtype, int D, int BQ, hipStream_t stream);
 
+// Few query rows against a long K/V (decode): one Q tile of Sq <= 32 rows per (b, h), its list of KV tiles split
+// over `nsplit` workgroups whose partial results a second kernel merges.
+struct DecodeParams {
+    const uint16_t *q, *k, *v;
+    uint16_t *o;
+    const uint8_t *mask;
+    const int32_t *full_ids, *full_lens, *part_ids, *part_lens;
+    int64_t qs[3], ks[3], vs[3], os[3];  // b, h, s strides in elements (d stride is 1)
+    int64_t ms[4];                        // mask strides in bytes
+    int64_t fis[3], fls[2], pis[3], pls[2];  // b, h (and entry) strides of the lists of the one Q tile
+    int B, H, Sq, Sk;
+    int BK, lbk;    // KV tile width (a power of two >= 32) and its log2
+    int mask_vec4;  // 1: mask columns are contiguous and 4-byte aligned
+    int nsplit;     // workgroups per (b, h)
+    float *ws;      // [B*H][nsplit][Sq][D + 2] floats: unnormalised rows, then reference value and row sum
+    float scale;    // softmax scale / ln 2
+};
+hipError_t launch_decode(const DecodeParams &p, int dtype, int D, hipStream_t stream);
+
 }  // namespace sa

@@ -31,14 +31,6 @@ namespace sa {
 
 namespace {
 
-template <int N, class F>
-__device__ __forceinline__ void static_for(F &&f) {  // f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)
-    if constexpr (N > 0) {
-        static_for<N - 1>(f);
-        f(std::integral_constant<int, N - 1>{});
-    }
-}
-
 // "At most n vector-memory operations of this wave still in flight", n a small run-time value.
 __device__ __forceinline__ void wait_vm_at_most(int n, int step) {
     if (n <= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

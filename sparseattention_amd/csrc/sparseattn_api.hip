@@ -419,4 +419,115 @@ int sa_mask_pack_partial(const uint8_t *mask, const int64_t mask_strides[4], int
     return SA_OK;
 }
 
+int sa_decode_num_splits(int B, int H, int Sq, int Sk, int BK) {
+    if (B <= 0 || H <= 0 || Sq <= 0 || Sq > 32 || Sk <= 0 || BK < 32 || Sk % BK) return 0;
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    // two workgroups per compute unit over all (b, h), at least eight 32-key chunks per workgroup
+    const int64_t bh = (int64_t)B * H;
+    int64_t n = (2 * (int64_t)cus + bh - 1) / bh;
+    const int64_t most = Sk / 256 > 0 ? Sk / 256 : 1;
+    if (n > most) n = most;
+    if (n > 256) n = 256;
+    if (n < 1) n = 1;
+    return (int)n;
+}
+
+size_t sa_decode_workspace_bytes(int B, int H, int Sq, int D, int num_splits) {
+    if (B <= 0 || H <= 0 || Sq <= 0 || D <= 0 || num_splits <= 1) return 0;
+    return (size_t)B * H * num_splits * Sq * (size_t)(D + 2) * sizeof(float);
+}
+
+int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                               const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
+                               const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
+                               const int64_t full_ids_strides[4], const int32_t *full_lens,
+                               const int64_t full_lens_strides[3], const int32_t *part_ids,
+                               const int64_t part_ids_strides[4], const int32_t *part_lens,
+                               const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int D, int BK,
+                               int dtype, float sm_scale_log2, int num_splits, void *workspace, size_t workspace_bytes,
+                               void *stream) {
+    g_error[0] = 0;
+    if (!q || !k || !v || !o || !q_strides || !k_strides || !v_strides || !o_strides || !mask || !mask_strides ||
+        !full_ids || !full_ids_strides || !full_lens || !full_lens_strides || !part_ids || !part_ids_strides ||
+        !part_lens || !part_lens_strides)
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_decode: null pointer argument");
+    if (const int rc = check_tiling(B, H, Sq, Sk, Sq > 0 ? Sq : 1, BK)) return rc;
+    if (Sq > 32) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_decode: Sq %d (supported: 1..32 query rows)", Sq);
+    if (D != 64 && D != 128) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_decode: head dim %d (supported: 64, 128)", D);
+    if (!(sm_scale_log2 > 0.f) || !(sm_scale_log2 < 3.0e38f))
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_decode: sm_scale_log2 must be positive and finite");
+    if (dtype != SA_DTYPE_BF16 && dtype != SA_DTYPE_FP16)
+        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_decode: dtype code %d (supported: 0 = bf16, 1 = fp16)", dtype);
+    const int lbk = log2_exact(BK);
+    if (lbk < 5) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_decode: BLOCK_K %d (supported: powers of two >= 32)", BK);
+    const int64_t *st[4] = {q_strides, k_strides, v_strides, o_strides};
+    const void *ptr[4] = {q, k, v, o};
+    const char *name[4] = {"q", "k", "v", "o"};
+    for (int t = 0; t < 4; t++) {
+        if (st[t][3] != 1)
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_decode: %s must be contiguous in its last dimension (stride %lld)", name[t], (long long)st[t][3]);
+        if (!aligned(ptr[t], 16) || st[t][0] % 8 || st[t][1] % 8 || st[t][2] % 8)
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_decode: %s needs a 16-byte aligned base and strides that are multiples of 8 elements", name[t]);
+    }
+    if ((Sq > 1 && o_strides[2] == 0) || (B > 1 && o_strides[0] == 0) || (H > 1 && o_strides[1] == 0))
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_decode: o must not alias itself (zero stride)");
+    if ((int64_t)B * H > 65535) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_decode: more than 65535 (b, h) planes");
+    if (num_splits == 0) num_splits = sa_decode_num_splits(B, H, Sq, Sk, BK);
+    if (num_splits < 1 || num_splits > 256)
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_decode: num_splits %d (1..256, or 0 for the default)", num_splits);
+    if ((int64_t)(Sk / 32) * num_splits > 0x7fffffffLL)
+        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_decode: Sk / 32 * num_splits exceeds 2^31-1");
+    const size_t need = sa_decode_workspace_bytes(B, H, Sq, D, num_splits);
+    if (need != 0 && (!workspace || workspace_bytes < need || !aligned(workspace, 16)))
+        return fail(SA_ERR_WORKSPACE, "sa_sparse_attention_decode: 16-byte aligned workspace of %zu bytes required, %zu given", need,
+                    workspace ? workspace_bytes : (size_t)0);
+
+    sa::DecodeParams dp{};
+    dp.q = static_cast<const uint16_t *>(q);
+    dp.k = static_cast<const uint16_t *>(k);
+    dp.v = static_cast<const uint16_t *>(v);
+    dp.o = static_cast<uint16_t *>(o);
+    dp.mask = mask;
+    dp.full_ids = full_ids;
+    dp.full_lens = full_lens;
+    dp.part_ids = part_ids;
+    dp.part_lens = part_lens;
+    for (int i = 0; i < 3; i++) {
+        dp.qs[i] = q_strides[i];
+        dp.ks[i] = k_strides[i];
+        dp.vs[i] = v_strides[i];
+        dp.os[i] = o_strides[i];
+    }
+    for (int i = 0; i < 4; i++) dp.ms[i] = mask_strides[i];
+    // the lists of the one Q tile: b and h strides, and the stride along the entries
+    dp.fis[0] = full_ids_strides[0];
+    dp.fis[1] = full_ids_strides[1];
+    dp.fis[2] = full_ids_strides[3];
+    dp.pis[0] = part_ids_strides[0];
+    dp.pis[1] = part_ids_strides[1];
+    dp.pis[2] = part_ids_strides[3];
+    dp.fls[0] = full_lens_strides[0];
+    dp.fls[1] = full_lens_strides[1];
+    dp.pls[0] = part_lens_strides[0];
+    dp.pls[1] = part_lens_strides[1];
+    dp.B = B;
+    dp.H = H;
+    dp.Sq = Sq;
+    dp.Sk = Sk;
+    dp.BK = BK;
+    dp.lbk = lbk;
+    dp.mask_vec4 = (mask_strides[3] == 1 && aligned(mask, 4) && mask_strides[0] % 4 == 0 && mask_strides[1] % 4 == 0 &&
+                    mask_strides[2] % 4 == 0)
+                       ? 1
+                       : 0;
+    dp.nsplit = num_splits;
+    dp.ws = static_cast<float *>(workspace);
+    dp.scale = sm_scale_log2;
+    const hipError_t e = sa::launch_decode(dp, dtype, D, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_decode: launch failed: %s", hipGetErrorString(e));
+    return SA_OK;
+}
+
 }  // extern "C"

@@ -37,6 +37,10 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
         raise RuntimeError("sparse_attention needs q, k, v on a ROCm GPU; there is no CPU path")
     if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
         raise TypeError(f"q, k, v must share dtype bfloat16 or float16 (got {q.dtype}, {k.dtype}, {v.dtype})")
+    if (Sq == BLOCK_Q and Sq < 32 and BLOCK_K >= 32 and getattr(mask_metadata, "packed_masks", None) is None
+            and getattr(mask_metadata, "schedule", None) is None):
+        # one Q tile of fewer rows than the forward kernels tile by: the split-KV kernels
+        return sparse_attention_decode(q, k, v, mask, BLOCK_K, mask_metadata)
     sm_scale = D ** (-0.5) * 1 / math.log(2)  # exp2 replaces exp (sparse_attn_kernel.py:152)
 
     mask = mask.expand(B, H, Sq, Sk)
@@ -84,5 +88,58 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
             rc = lib.sa_sparse_attention_fwd_ex(*common, *pk, *sc, *tail)
         else:
             rc = lib.sa_sparse_attention_fwd(*common, *tail)
+    _native.check(rc)
+    return o
+
+
+def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor, BLOCK_K,
+                            mask_metadata: MaskMetadata | None = None, num_splits: int = 0) -> torch.Tensor:
+    """:func:`sparse_attention` for Sq <= 32 query rows (decode, speculative or chunked-prefill tails), BLOCK_Q = Sq.
+
+    The reference lists decode kernels as future work (README.md:65); the result is defined by its forward
+    (sparse_attn_kernel.py:149-185) called with ``BLOCK_Q = Sq``.  Every (b, h) has one Q tile, so its list of KV
+    tiles is cut into ``num_splits`` ranges (0: chosen from the shape and the device) that run in parallel and are
+    merged afterwards.  ``mask_metadata``: from ``compute_mask_kernel(mask, Sq, BLOCK_K)``.
+    """
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("q, k, v must be [B,H,S,D]")
+    B, H, Sq, D = q.shape
+    Sk = k.shape[-2]
+    if k.shape != (B, H, Sk, D) or v.shape != (B, H, Sk, D):
+        raise ValueError(f"k/v shapes {tuple(k.shape)}/{tuple(v.shape)} do not match q {tuple(q.shape)}")
+    if not q.is_cuda:
+        raise RuntimeError("sparse_attention_decode needs q, k, v on a ROCm GPU; there is no CPU path")
+    if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise TypeError(f"q, k, v must share dtype bfloat16 or float16 (got {q.dtype}, {k.dtype}, {v.dtype})")
+    sm_scale = D ** (-0.5) * 1 / math.log(2)
+    mask = mask.expand(B, H, Sq, Sk)
+    if mask_metadata is None:
+        mask_metadata = compute_mask_kernel(mask, Sq, BLOCK_K)
+    fid, fl = mask_metadata.unmasked_kv_ids, mask_metadata.unmasked_lens
+    pid, pl = mask_metadata.masked_kv_ids, mask_metadata.masked_lens
+    nK = Sk // BLOCK_K
+    for name, t, shape in (("unmasked_kv_ids", fid, (B, H, 1, nK)), ("masked_kv_ids", pid, (B, H, 1, nK)),
+                           ("unmasked_lens", fl, (B, H, 1)), ("masked_lens", pl, (B, H, 1))):
+        if tuple(t.shape) != shape or t.dtype != torch.int32 or t.device != q.device:
+            raise ValueError(f"mask_metadata.{name}: expected int32 {shape} on {q.device}, got {t.dtype} {tuple(t.shape)} on {t.device}")
+    assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
+    if mask.device != q.device:
+        raise ValueError("mask must be on the same device as q")
+    qc, kc, vc = _kernel_ready(q), _kernel_ready(k), _kernel_ready(v)
+    o = torch.empty_like(qc)
+    lib = _native.load()
+    S = _native.strides
+    with torch.cuda.device(q.device):
+        if num_splits == 0:
+            num_splits = lib.sa_decode_num_splits(B, H, Sq, Sk, int(BLOCK_K))
+        ws_bytes = lib.sa_decode_workspace_bytes(B, H, Sq, D, int(num_splits))
+        ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=q.device) if ws_bytes else None
+        rc = lib.sa_sparse_attention_decode(
+            qc.data_ptr(), S(qc.stride()), kc.data_ptr(), S(kc.stride()), vc.data_ptr(), S(vc.stride()),
+            o.data_ptr(), S(o.stride()), mask.data_ptr(), S(mask.stride()),
+            fid.data_ptr(), S(fid.stride()), fl.data_ptr(), S(fl.stride()),
+            pid.data_ptr(), S(pid.stride()), pl.data_ptr(), S(pl.stride()),
+            B, H, Sq, Sk, D, int(BLOCK_K), _DTYPES[q.dtype], sm_scale, int(num_splits),
+            ws.data_ptr() if ws is not None else None, ws_bytes, torch.cuda.current_stream(q.device).cuda_stream)
     _native.check(rc)
     return o
