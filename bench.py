@@ -17,6 +17,8 @@ the reference also excludes preprocessing from the forward time and reports it s
   across_p   the same forward on random block masks of sparsity p, a dense mask and the causal one
   variants   the headline workload through the other routes of the library (bool-mask reads, no schedule,
              persistent workgroups)
+  decode     the split-KV kernels for few query rows (sparse_attention_decode) against the HBM peak: K and V of
+             the executed tiles are read once
   cpu_baseline / cpu_sdpa_baseline   the CPU oracle and torch's masked SDPA on a bounded sample
 """
 import argparse
@@ -37,6 +39,8 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E peak, GB/s
 # are profiles/sparse_fwd_kernel_causal_B8H32S4096D128.txt and profiles/mask_classify_kernels_mask_32768x32768.txt.
 TRAFFIC_FWD_CAUSAL_BYTES = 1.3566e9      # 1037.8 MiB read + 256.0 MiB written
 TRAFFIC_CLASSIFY_1GIB_BYTES = 1.0744e9   # 1,048,622 + 327 KiB read, 256 + 45.5 KiB written
+# decode workloads (profiles/sparse_decode_kernel_B8H32Sk32768D128.txt), both kernels
+TRAFFIC_DECODE_BYTES = (4.2959e9, 1.6225e9)
 
 B, H, S, D = 8, 32, 4096, 128
 BQ, BK = 128, 32
@@ -51,6 +55,7 @@ def parse():
     ap.add_argument("--no-sweep", action="store_true", help="skip the across-p table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--no-classify", action="store_true", help="skip the mask-classification timing")
+    ap.add_argument("--no-decode", action="store_true", help="skip the few-query-rows (decode) timing")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy a few times, so that a counter run over this command "
                          "holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -160,6 +165,44 @@ def classify_small_case(steps, warmup):
     _, full_ms = time_launches(lambda: compute_mask_kernel(me, BQ, BK, schedule="pairs"), steps, warmup)
     return {"workload": "compute_mask_kernel on the causal mask [4096,4096] = 16 MiB (latency bound)",
             "ms": round(ev_ms, 4), "with_pack_and_schedule_ms": round(full_ms, 4)}
+
+
+def decode_case(steps, warmup):
+    """Few query rows against a 32k context (B8 H32 D128 bf16, KV tiles of 128): HBM-bound."""
+    import torch
+    from sparseattention_amd import compute_mask_kernel, sparse_attention_decode, workloads as W
+
+    Sk, BKd = 32768, 128
+    rows = []
+    k = v = None
+    for case, (name, Sq) in enumerate((("1 query row, every key", 1),
+                                       ("16 query rows, causal window 4096 + 512 sink keys + 25% of the far tiles", 16))):
+        q, k2, v2 = W.qkv(B, H, Sq, D, torch.bfloat16, seed=1, device="cuda", Sk=Sk)
+        if k is None:
+            k, v = k2, v2
+        del k2, v2
+        if Sq == 1:
+            mask = torch.ones(Sq, Sk, dtype=torch.bool, device="cuda")
+        else:
+            pos_q = torch.arange(Sk - Sq, Sk, device="cuda")[:, None]
+            pos_k = torch.arange(Sk, device="cuda")[None, :]
+            far = (torch.rand(Sk // BKd, generator=torch.Generator().manual_seed(2)) < 0.25).to("cuda").repeat_interleave(BKd)
+            mask = (pos_k <= pos_q) & ((pos_q - pos_k < 4096) | (pos_k < 512) | far[None, :])
+        me = mask.expand(B, H, Sq, Sk)
+        md = compute_mask_kernel(me, Sq, BKd)
+        tiles = int(md.unmasked_lens.sum()) + int(md.masked_lens.sum())
+        nbytes = tiles * BKd * D * 2 * 2 + 2 * B * H * Sq * D * 2  # K and V rows of the executed tiles, q read, o written
+        wall_ms, ev_ms = time_launches(lambda: sparse_attention_decode(q, k, v, me, BKd, mask_metadata=md), steps, warmup)
+        rows.append({
+            "workload": f"{name}; Sk=32768, B=8 H=32 D=128 bf16, BLOCK_K=128",
+            "executed_tile_fraction": round(tiles / (B * H * (Sk // BKd)), 5),
+            "ms": round(wall_ms, 4), "kernel_ms": round(ev_ms, 4),
+            "roofline": {"bound": "hbm", "achieved": round(nbytes / (ev_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": round(nbytes / (ev_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                         "traffic": TRAFFIC_DECODE_BYTES[case], "algorithmic_bytes": nbytes,
+                         "kernel": "sparse_decode_kernel (+ decode_merge_kernel)"},
+        })
+    return rows
 
 
 def cpu_baselines():
@@ -275,6 +318,8 @@ def main():
         result["mask_classify"] = classify_case(max(10, args.steps // 2), max(3, args.warmup // 2))
         result["mask_classify_headline"] = classify_small_case(max(10, args.steps // 2), max(3, args.warmup // 2))
     del q, k, v
+    if not args.no_decode:
+        result["decode"] = decode_case(max(10, args.steps // 2), max(3, args.warmup // 2))
     if args.calibrate_copy:
         src = torch.ones(1 << 28, dtype=torch.int32, device="cuda")  # 1 GiB read + 1 GiB written per copy
         dst = torch.empty_like(src)
