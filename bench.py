@@ -22,6 +22,7 @@ the reference also excludes preprocessing from the forward time and reports it s
   cpu_baseline / cpu_sdpa_baseline   the CPU oracle and torch's masked SDPA on a bounded sample
 """
 import argparse
+import gc
 import json
 import math
 import os
@@ -71,14 +72,21 @@ def time_launches(fn, steps, warmup):
         fn()
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        starts[i].record()
-        fn()
-        ends[i].record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    # a collection of the interpreter's cyclic garbage inside the timed region costs tens of milliseconds of host
+    # time, which a microsecond-scale step would report as its own
+    gc.collect()
+    gc.disable()
+    try:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            starts[i].record()
+            fn()
+            ends[i].record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    finally:
+        gc.enable()
     ev_ms = sum(s.elapsed_time(e) for s, e in zip(starts, ends)) / steps
     return wall_ms, ev_ms
 
