@@ -143,5 +143,19 @@ __device__ __forceinline__ void static_for(F &&f) {  // f(integral_constant<int,
     }
 }
 
+// Raises a kernel's dynamic shared-memory limit to `bytes`, once per device: `done` is the caller's bit mask of the
+// devices (ordinals below 64) that have it.  Two threads racing here set the same value twice.
+template <class K>
+hipError_t allow_dynamic_smem(K kern, int bytes, unsigned long long &done) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const unsigned long long bit = dev >= 0 && dev < 64 ? 1ull << dev : 0ull;
+    if (bit != 0 && (__atomic_load_n(&done, __ATOMIC_RELAXED) & bit)) return hipSuccess;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess && bit != 0) __atomic_fetch_or(&done, bit, __ATOMIC_RELAXED);
+    return e;
+}
+
 }  // namespace
 }  // namespace sa

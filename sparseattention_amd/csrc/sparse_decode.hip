@@ -312,13 +312,8 @@ template <int DT, int D>
 hipError_t launch_decode_one(const DecodeParams &p, hipStream_t stream) {
     constexpr int smem = decode_smem_bytes<D>();
     auto kern = sparse_decode_kernel<DT, D>;
-    static bool attr_set = false;  // benign race: every thread sets the same value
-    if (!attr_set) {
-        const hipError_t e =
-            hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static unsigned long long attr_done = 0;  // devices on which this kernel may use `smem` bytes of LDS
+    if (const hipError_t e0 = allow_dynamic_smem(kern, smem, attr_done); e0 != hipSuccess) return e0;
     hipLaunchKernelGGL(kern, dim3(p.nsplit, p.B * p.H), dim3(kDecodeWaves * 64), smem, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || p.nsplit == 1) return e;

@@ -957,13 +957,8 @@ hipError_t launch_one(const FwdParams &p, hipStream_t stream) {
     static_assert(kListCap == 2 * kPsListCap, "one long list or two short ones in the same LDS");
     constexpr int smem = 2 * NS * 64 * D * 2 + kListCap * 4;  // NS stages of 64 rows for K and for V + the list(s)
     auto kern = sparse_fwd_kernel<DT, D, NW, MODE, NS, NW == 8, PK, PS>;
-    static bool attr_set = false;  // benign race: every thread sets the same value
-    if (!attr_set) {
-        const hipError_t e =
-            hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static unsigned long long attr_done = 0;  // devices on which this kernel may use `smem` bytes of LDS
+    if (const hipError_t e0 = allow_dynamic_smem(kern, smem, attr_done); e0 != hipSuccess) return e0;
     const unsigned grid = PS ? (unsigned)p.sched_G : (unsigned)p.nQ * (unsigned)p.B * (unsigned)p.H;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), smem, stream, p);
     return hipGetLastError();
