@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define SA_ABI_VERSION 5
+#define SA_ABI_VERSION 6
 
 enum sa_status {
     SA_OK = 0,
@@ -198,6 +198,24 @@ int sa_sparse_attention_fwd_ex(const void *q, const int64_t q_strides[4], const 
                                float sm_scale_log2, void *stream);
 
 /*
+ * sa_sparse_attention_fwd_ex with a second output: lse[b,h,row] = ln sum over the attended keys of
+ * exp(q.k * softmax scale), float32, -inf for rows that attend to nothing (what a caller needs to merge results
+ * over disjoint key ranges, or to run a backward pass; the reference keeps the row maximum and sum in registers,
+ * sparse_attn_kernel.py:107-108, and drops them after the division at :144).  lse, lse_strides (elements; b, h,
+ * row) may be NULL: then this is sa_sparse_attention_fwd_ex.  `o` is bit-identical either way.
+ */
+int sa_sparse_attention_fwd_lse(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                                const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
+                                const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
+                                const int64_t full_ids_strides[4], const int32_t *full_lens,
+                                const int64_t full_lens_strides[3], const int32_t *part_ids,
+                                const int64_t part_ids_strides[4], const int32_t *part_lens,
+                                const int64_t part_lens_strides[3], const uint8_t *packed,
+                                const int64_t packed_strides[2], const int32_t *schedule, size_t schedule_bytes,
+                                int schedule_mode, float *lse, const int64_t lse_strides[3], int B, int H, int Sq,
+                                int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2, void *stream);
+
+/*
  * The forward for few query rows against a long K/V (decode): Sq <= 32 rows form the single Q tile of every (b, h),
  * BLOCK_Q = Sq.  The result is that of sparse_attention (sparseattention/sparse_attn_kernel.py:149-185) called with
  * BLOCK_Q = Sq; the reference has no kernel of its own for this shape ("Backwards pass + decode kernels" is item 3
@@ -211,6 +229,7 @@ int sa_sparse_attention_fwd_ex(const void *q, const int64_t q_strides[4], const 
  *   num_splits   workgroups per (b, h), 1..256, or 0 for sa_decode_num_splits(...)
  *   workspace    sa_decode_workspace_bytes(...) bytes of device memory, 16-byte aligned (may be NULL when that is 0,
  *                i.e. for one split); contents on return are unspecified
+ *   lse, lse_strides   optional second output as in sa_sparse_attention_fwd_lse, or NULL
  * q, k, v, o, D, dtype, sm_scale_log2, stream: as for sa_sparse_attention_fwd.
  */
 int sa_decode_num_splits(int B, int H, int Sq, int Sk, int BK);
@@ -223,7 +242,7 @@ int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const 
                                const int64_t part_ids_strides[4], const int32_t *part_lens,
                                const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int D, int BK,
                                int dtype, float sm_scale_log2, int num_splits, void *workspace, size_t workspace_bytes,
-                               void *stream);
+                               float *lse, const int64_t lse_strides[3], void *stream);
 
 #ifdef __cplusplus
 }

@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsparseattn_hip.so")
 
-SA_ABI_VERSION = 5
+SA_ABI_VERSION = 6
 SA_OK = 0
 SA_ERR_INVALID_ARGUMENT = -1
 SA_ERR_UNSUPPORTED = -2
@@ -35,6 +35,7 @@ EXPORTS = (
     "sa_fwd_schedule_bytes",
     "sa_fwd_schedule",
     "sa_sparse_attention_fwd_ex",
+    "sa_sparse_attention_fwd_lse",
     "sa_decode_num_splits",
     "sa_decode_workspace_bytes",
     "sa_sparse_attention_decode",
@@ -92,6 +93,11 @@ def load() -> ctypes.CDLL:
         [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, ctypes.c_size_t]
         + [ctypes.c_int] * 9 + [ctypes.c_float, _vp]
     )
+    lib.sa_sparse_attention_fwd_lse.restype = ctypes.c_int
+    lib.sa_sparse_attention_fwd_lse.argtypes = (
+        [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, ctypes.c_size_t, ctypes.c_int]
+        + [_vp, _i64p] + [ctypes.c_int] * 8 + [ctypes.c_float, _vp]
+    )
     lib.sa_decode_num_splits.restype = ctypes.c_int
     lib.sa_decode_num_splits.argtypes = [ctypes.c_int] * 5
     lib.sa_decode_workspace_bytes.restype = ctypes.c_size_t
@@ -99,7 +105,7 @@ def load() -> ctypes.CDLL:
     lib.sa_sparse_attention_decode.restype = ctypes.c_int
     lib.sa_sparse_attention_decode.argtypes = (
         [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [ctypes.c_int] * 7 + [ctypes.c_float, ctypes.c_int]
-        + [_vp, ctypes.c_size_t, _vp]
+        + [_vp, ctypes.c_size_t] + [_vp, _i64p] + [_vp]
     )
     if lib.sa_abi_version() != SA_ABI_VERSION:
         raise RuntimeError(f"libsparseattn_hip ABI {lib.sa_abi_version()} != expected {SA_ABI_VERSION}")

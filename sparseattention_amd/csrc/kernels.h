@@ -79,6 +79,10 @@ struct FwdParams {
     const int32_t *sched;
     int sched_G, sched_R;  // workgroups, and entries per row after the header entry
     float scale;    // softmax scale / ln 2
+    // Optional second output: natural-log sum of exp(scaled score) over the attended keys of every query row
+    // (-inf for rows without one), or null.
+    float *lse;
+    int64_t lses[3];  // b, h, row strides in elements
 };
 
 // dtype: 0 bf16, 1 fp16.  Returns hipErrorInvalidValue when no instantiation matches (D, BQ).
@@ -100,6 +104,8 @@ struct DecodeParams {
     int nsplit;     // workgroups per (b, h)
     float *ws;      // [B*H][nsplit][Sq][D + 2] floats: unnormalised rows, then reference value and row sum
     float scale;    // softmax scale / ln 2
+    float *lse;     // optional second output as in FwdParams, or null
+    int64_t lses[3];
 };
 hipError_t launch_decode(const DecodeParams &p, int dtype, int D, hipStream_t stream);
 

@@ -275,6 +275,9 @@ __global__ __launch_bounds__(kDecodeWaves * 64, 2) void sparse_decode_kernel(con
             merge_parts<NV>(part + q * PST, kDecodeWaves, 32 * PST, D, d0, out, M, L);
             if (p.nsplit == 1) {
                 const float inv = L > 0.f ? 1.f / L : 0.f;
+                if (p.lse != nullptr && (tid & 7) == 0)
+                    p.lse[b * p.lses[0] + h * p.lses[1] + q * p.lses[2]] =
+                        L > 0.f ? (M + __builtin_amdgcn_logf(L)) * 0.69314718056f : kNegInf;
                 uint16_t *orow = p.o + b * p.os[0] + h * p.os[1] + (int64_t)q * p.os[2] + d0;
 #pragma unroll
                 for (int j = 0; j < NV; j += 2) *(uint32_t *)(orow + j) = E::pack2(out[j] * inv, out[j + 1] * inv);
@@ -303,6 +306,9 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(const DecodeParams p)
     float out[NV], M, L;
     merge_parts<NV>(p.ws + ((int64_t)bh * p.nsplit * p.Sq + q) * PST, p.nsplit, (int64_t)p.Sq * PST, D, d0, out, M, L);
     const float inv = L > 0.f ? 1.f / L : 0.f;
+    if (p.lse != nullptr && (tid & 7) == 0)
+        p.lse[b * p.lses[0] + h * p.lses[1] + q * p.lses[2]] =
+            L > 0.f ? (M + __builtin_amdgcn_logf(L)) * 0.69314718056f : kNegInf;
     uint16_t *orow = p.o + b * p.os[0] + h * p.os[1] + (int64_t)q * p.os[2] + d0;
 #pragma unroll
     for (int j = 0; j < NV; j += 2) *(uint32_t *)(orow + j) = E::pack2(out[j] * inv, out[j + 1] * inv);

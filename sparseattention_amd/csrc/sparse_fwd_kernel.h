@@ -91,6 +91,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
     const uint8_t *mrow, *prow;
     const int32_t *fid, *pid;
     int64_t orow_off;  // this lane's first output element
+    int64_t lse_off;   // this lane's row in p.lse
     // this lane's row in a packed tile: BK/8 bytes per row, NW*32 rows per tile
     const int64_t tile_bytes = (int64_t)(NW * 4) * p.BK;
     const int sh4 = 4 * hh;
@@ -132,6 +133,7 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         pid = p.part_ids + b * p.pis[0] + h * p.pis[1] + qt * p.pis[2];
         const int qrow_ = qt * (NW * 32) + wave * 32 + l32;
         orow_off = b * p.os[0] + h * p.os[1] + (int64_t)qrow_ * p.os[2] + 4 * hh;
+        lse_off = b * p.lses[0] + h * p.lses[1] + (int64_t)qrow_ * p.lses[2];
     };
     // Row of this workgroup in the schedule: entry 0 = {number of Q tiles, -, -, -}, then one entry
     // {(b << 16) | h, qt, F, P} per Q tile.
@@ -615,6 +617,9 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
     auto store_o = [&]() {
         const float l_tot = l32 < 16 ? acc_l[0] : acc_l[1];
         const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        // sum over the attended keys of exp(scaled score) = l * 2^m_ref
+        if (p.lse != nullptr && hh == 0)
+            p.lse[lse_off] = l_tot > 0.f ? (m_ref + __builtin_amdgcn_logf(l_tot)) * 0.69314718056f : kNegInf;
         uint16_t *orow = p.o + orow_off;
 #pragma unroll
         for (int db = 0; db < D / 32; db++)

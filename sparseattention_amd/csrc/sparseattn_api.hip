@@ -180,8 +180,8 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
                  const int32_t *full_lens, const int64_t full_lens_strides[3], const int32_t *part_ids,
                  const int64_t part_ids_strides[4], const int32_t *part_lens, const int64_t part_lens_strides[3],
                  const uint8_t *packed, const int64_t packed_strides[2], bool use_packed, const int32_t *schedule,
-                 size_t schedule_bytes, int schedule_mode, int B, int H, int Sq, int Sk, int D, int BQ, int BK,
-                 int dtype, float sm_scale_log2, void *stream) {
+                 size_t schedule_bytes, int schedule_mode, float *lse, const int64_t lse_strides[3], int B, int H,
+                 int Sq, int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2, void *stream) {
     g_error[0] = 0;
     if (!q || !k || !v || !o || !q_strides || !k_strides || !v_strides || !o_strides || !full_ids ||
         !full_ids_strides || !full_lens || !full_lens_strides || !part_ids || !part_ids_strides || !part_lens ||
@@ -266,6 +266,14 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
                        ? 1
                        : 0;
     fp.scale = sm_scale_log2;
+    fp.lse = nullptr;
+    if (lse) {
+        if (!lse_strides) return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd_lse: null pointer argument (lse_strides)");
+        if (!aligned(lse, 4) || (Sq > 1 && lse_strides[2] == 0) || (B > 1 && lse_strides[0] == 0) || (H > 1 && lse_strides[1] == 0))
+            return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd_lse: lse must be 4-byte aligned and must not alias itself (zero stride)");
+        fp.lse = lse;
+        for (int i = 0; i < 3; i++) fp.lses[i] = lse_strides[i];
+    }
     const hipError_t e = sa::launch_fwd(fp, dtype, D, BQ, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_fwd: launch failed: %s", hipGetErrorString(e));
     return SA_OK;
@@ -299,8 +307,8 @@ int sa_sparse_attention_fwd(const void *q, const int64_t q_strides[4], const voi
                             int dtype, float sm_scale_log2, void *stream) {
     return forward_impl(q, q_strides, k, k_strides, v, v_strides, o, o_strides, mask, mask_strides, full_ids,
                         full_ids_strides, full_lens, full_lens_strides, part_ids, part_ids_strides, part_lens,
-                        part_lens_strides, nullptr, nullptr, false, nullptr, 0, 0, B, H, Sq, Sk, D, BQ, BK, dtype,
-                        sm_scale_log2, stream);
+                        part_lens_strides, nullptr, nullptr, false, nullptr, 0, 0, nullptr, nullptr, B, H, Sq, Sk, D, BQ,
+                        BK, dtype, sm_scale_log2, stream);
 }
 
 int sa_sparse_attention_fwd_ex(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
@@ -323,7 +331,30 @@ int sa_sparse_attention_fwd_ex(const void *q, const int64_t q_strides[4], const 
     return forward_impl(q, q_strides, k, k_strides, v, v_strides, o, o_strides, mask, mask_strides, full_ids,
                         full_ids_strides, full_lens, full_lens_strides, part_ids, part_ids_strides, part_lens,
                         part_lens_strides, packed, packed_strides, use_packed, schedule, schedule_bytes, schedule_mode,
-                        B, H, Sq, Sk, D, BQ, BK, dtype, sm_scale_log2, stream);
+                        nullptr, nullptr, B, H, Sq, Sk, D, BQ, BK, dtype, sm_scale_log2, stream);
+}
+
+int sa_sparse_attention_fwd_lse(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                                const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
+                                const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
+                                const int64_t full_ids_strides[4], const int32_t *full_lens,
+                                const int64_t full_lens_strides[3], const int32_t *part_ids,
+                                const int64_t part_ids_strides[4], const int32_t *part_lens,
+                                const int64_t part_lens_strides[3], const uint8_t *packed,
+                                const int64_t packed_strides[2], const int32_t *schedule, size_t schedule_bytes,
+                                int schedule_mode, float *lse, const int64_t lse_strides[3], int B, int H, int Sq,
+                                int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2, void *stream) {
+    const bool use_packed = packed != nullptr;
+    if (use_packed) {
+        g_error[0] = 0;
+        if (!packed_strides) return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd_lse: null pointer argument (packed_strides)");
+        if ((B > 1 && packed_strides[0] % 4) || (H > 1 && packed_strides[1] % 4) || !aligned(packed, 4))
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd_lse: packed needs a 4-byte aligned base and plane strides");
+    }
+    return forward_impl(q, q_strides, k, k_strides, v, v_strides, o, o_strides, mask, mask_strides, full_ids,
+                        full_ids_strides, full_lens, full_lens_strides, part_ids, part_ids_strides, part_lens,
+                        part_lens_strides, packed, packed_strides, use_packed, schedule, schedule_bytes, schedule_mode,
+                        lse, lse_strides, B, H, Sq, Sk, D, BQ, BK, dtype, sm_scale_log2, stream);
 }
 
 size_t sa_fwd_schedule_bytes(int B, int H, int Sq, int Sk, int BQ, int BK, int mode) {
@@ -447,7 +478,7 @@ int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const 
                                const int64_t part_ids_strides[4], const int32_t *part_lens,
                                const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int D, int BK,
                                int dtype, float sm_scale_log2, int num_splits, void *workspace, size_t workspace_bytes,
-                               void *stream) {
+                               float *lse, const int64_t lse_strides[3], void *stream) {
     g_error[0] = 0;
     if (!q || !k || !v || !o || !q_strides || !k_strides || !v_strides || !o_strides || !mask || !mask_strides ||
         !full_ids || !full_ids_strides || !full_lens || !full_lens_strides || !part_ids || !part_ids_strides ||
@@ -525,6 +556,14 @@ int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const 
     dp.nsplit = num_splits;
     dp.ws = static_cast<float *>(workspace);
     dp.scale = sm_scale_log2;
+    dp.lse = nullptr;
+    if (lse) {
+        if (!lse_strides) return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_decode: null pointer argument (lse_strides)");
+        if (!aligned(lse, 4) || (Sq > 1 && lse_strides[2] == 0) || (B > 1 && lse_strides[0] == 0) || (H > 1 && lse_strides[1] == 0))
+            return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_decode: lse must be 4-byte aligned and must not alias itself (zero stride)");
+        dp.lse = lse;
+        for (int i = 0; i < 3; i++) dp.lses[i] = lse_strides[i];
+    }
     const hipError_t e = sa::launch_decode(dp, dtype, D, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_decode: launch failed: %s", hipGetErrorString(e));
     return SA_OK;

@@ -18,14 +18,16 @@ def _kernel_ready(t: torch.Tensor) -> torch.Tensor:
 
 
 def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor, BLOCK_Q, BLOCK_K,
-                     mask_metadata: MaskMetadata | None = None) -> torch.Tensor:
+                     mask_metadata: MaskMetadata | None = None, *, return_lse: bool = False):
     """softmax(q kᵀ / sqrt(D) + (mask ? 0 : -inf)) v, skipping KV tiles the mask empties.
 
     Signature and meaning follow sparse_attn_kernel.py:149-185: ``q`` [B,H,Sq,D], ``k``/``v``
     [B,H,Sk,D] (bf16 or fp16, on a ROCm GPU), ``mask`` bool broadcastable to [B,H,Sq,Sk] with
     True = attend, tile sizes ``BLOCK_Q`` x ``BLOCK_K``, and optionally the metadata from
     :func:`compute_mask_kernel` so that preprocessing is paid once for many calls.
-    Returns ``o`` with q's shape, dtype and strides.
+    Returns ``o`` with q's shape, dtype and strides; with ``return_lse=True`` (not in the reference, which drops
+    the row statistics after the division at sparse_attn_kernel.py:144) the pair ``(o, lse)`` where ``lse``
+    [B,H,Sq] float32 is the log of the row's softmax denominator, -inf for rows that attend to nothing.
     """
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be [B,H,S,D]")
@@ -40,7 +42,7 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
     if (Sq == BLOCK_Q and Sq < 32 and BLOCK_K >= 32 and getattr(mask_metadata, "packed_masks", None) is None
             and getattr(mask_metadata, "schedule", None) is None):
         # one Q tile of fewer rows than the forward kernels tile by: the split-KV kernels
-        return sparse_attention_decode(q, k, v, mask, BLOCK_K, mask_metadata)
+        return sparse_attention_decode(q, k, v, mask, BLOCK_K, mask_metadata, return_lse=return_lse)
     sm_scale = D ** (-0.5) * 1 / math.log(2)  # exp2 replaces exp (sparse_attn_kernel.py:152)
 
     mask = mask.expand(B, H, Sq, Sk)
@@ -81,25 +83,31 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
         tail = (B, H, Sq, Sk, D, int(BLOCK_Q), int(BLOCK_K), _DTYPES[q.dtype], sm_scale,
                 torch.cuda.current_stream(q.device).cuda_stream)
         sched = getattr(mask_metadata, "schedule", None)
-        if packed is not None or sched is not None:
+        lse = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device) if return_lse else None
+        if packed is not None or sched is not None or return_lse:
             pk = (packed.data_ptr(), S(packed.stride()[:2])) if packed is not None else (None, None)
             sc = ((sched.data_ptr(), sched.numel() * 4, int(getattr(mask_metadata, "schedule_mode", 0)))
                   if sched is not None else (None, 0, 0))
-            rc = lib.sa_sparse_attention_fwd_ex(*common, *pk, *sc, *tail)
+            if return_lse:
+                rc = lib.sa_sparse_attention_fwd_lse(*common, *pk, *sc, lse.data_ptr(), S(lse.stride()), *tail)
+            else:
+                rc = lib.sa_sparse_attention_fwd_ex(*common, *pk, *sc, *tail)
         else:
             rc = lib.sa_sparse_attention_fwd(*common, *tail)
     _native.check(rc)
-    return o
+    return (o, lse) if return_lse else o
 
 
 def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor, BLOCK_K,
-                            mask_metadata: MaskMetadata | None = None, num_splits: int = 0) -> torch.Tensor:
+                            mask_metadata: MaskMetadata | None = None, num_splits: int = 0, *,
+                            return_lse: bool = False):
     """:func:`sparse_attention` for Sq <= 32 query rows (decode, speculative or chunked-prefill tails), BLOCK_Q = Sq.
 
     The reference lists decode kernels as future work (README.md:65); the result is defined by its forward
     (sparse_attn_kernel.py:149-185) called with ``BLOCK_Q = Sq``.  Every (b, h) has one Q tile, so its list of KV
     tiles is cut into ``num_splits`` ranges (0: chosen from the shape and the device) that run in parallel and are
-    merged afterwards.  ``mask_metadata``: from ``compute_mask_kernel(mask, Sq, BLOCK_K)``.
+    merged afterwards.  ``mask_metadata``: from ``compute_mask_kernel(mask, Sq, BLOCK_K)``.  ``return_lse``: as in
+    :func:`sparse_attention`.
     """
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be [B,H,S,D]")
@@ -134,12 +142,15 @@ def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, m
             num_splits = lib.sa_decode_num_splits(B, H, Sq, Sk, int(BLOCK_K))
         ws_bytes = lib.sa_decode_workspace_bytes(B, H, Sq, D, int(num_splits))
         ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=q.device) if ws_bytes else None
+        lse = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device) if return_lse else None
         rc = lib.sa_sparse_attention_decode(
             qc.data_ptr(), S(qc.stride()), kc.data_ptr(), S(kc.stride()), vc.data_ptr(), S(vc.stride()),
             o.data_ptr(), S(o.stride()), mask.data_ptr(), S(mask.stride()),
             fid.data_ptr(), S(fid.stride()), fl.data_ptr(), S(fl.stride()),
             pid.data_ptr(), S(pid.stride()), pl.data_ptr(), S(pl.stride()),
             B, H, Sq, Sk, D, int(BLOCK_K), _DTYPES[q.dtype], sm_scale, int(num_splits),
-            ws.data_ptr() if ws is not None else None, ws_bytes, torch.cuda.current_stream(q.device).cuda_stream)
+            ws.data_ptr() if ws is not None else None, ws_bytes,
+            lse.data_ptr() if lse is not None else None, S(lse.stride()) if lse is not None else None,
+            torch.cuda.current_stream(q.device).cuda_stream)
     _native.check(rc)
-    return o
+    return (o, lse) if return_lse else o

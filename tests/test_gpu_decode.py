@@ -173,7 +173,29 @@ def test_errors(gpu):
         S(o.stride()), me.data_ptr(), S(me.stride()), md.unmasked_kv_ids.data_ptr(), S(md.unmasked_kv_ids.stride()),
         md.unmasked_lens.data_ptr(), S(md.unmasked_lens.stride()), md.masked_kv_ids.data_ptr(),
         S(md.masked_kv_ids.stride()), md.masked_lens.data_ptr(), S(md.masked_lens.stride()), B, H, 8, Sk, D, 32,
-        _native.SA_DTYPE_BF16, D ** -0.5 / math.log(2), 4, ws.data_ptr(), ws.numel() * 4,
+        _native.SA_DTYPE_BF16, D ** -0.5 / math.log(2), 4, ws.data_ptr(), ws.numel() * 4, None, None,
         ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
     assert rc == _native.SA_ERR_WORKSPACE and b"workspace" in lib.sa_last_error()
     assert 1 <= lib.sa_decode_num_splits(8, 32, 1, 32768, 128) <= 256
+
+
+def lse_fp64(q, k, mask):
+    s = torch.einsum("bhqd,bhkd->bhqk", q.double(), k.double()) / math.sqrt(q.shape[-1])
+    return torch.logsumexp(s.masked_fill(~mask.expand(s.shape), -math.inf), dim=-1)
+
+
+@pytest.mark.parametrize("splits", [1, 5])
+def test_lse_output(gpu, splits):
+    B, H, Sq, Sk, D, BK = 2, 2, 6, 2048, 128, 64
+    q, k, v = W.qkv(B, H, Sq, D, torch.bfloat16, seed=31, device=gpu, Sk=Sk)
+    mask = tile_mask((B, H, Sq, Sk), BK, seed=32, device=gpu, keep_first=False)
+    mask[1, 1, 3] = False
+    o, lse = sparse_attention_decode(q, k, v, mask, BK, num_splits=splits, return_lse=True)
+    assert torch.equal(o, sparse_attention_decode(q, k, v, mask, BK, num_splits=splits))
+    want = lse_fp64(q, k, mask)
+    assert lse.shape == (B, H, Sq) and lse.dtype == torch.float32
+    assert lse[1, 1, 3] == -math.inf and torch.isinf(want[1, 1, 3])
+    live = torch.isfinite(want)
+    assert torch.equal(live, torch.isfinite(lse))
+    # the row sum adds up P as rounded to bf16 for the P.V product: relative error of the sum below 2^-9
+    assert (lse[live].double() - want[live]).abs().max() <= 4e-3

@@ -282,3 +282,29 @@ def test_runs_on_a_side_stream(gpu):
         got = sparse_attention(q, k, v, mask, 128, 32)
     s.synchronize()
     assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("route", ["plain", "packed+pairs", "persistent"])
+@pytest.mark.parametrize("BQ,BK", [(128, 32), (64, 64), (256, 16)])
+def test_lse_output(gpu, route, BQ, BK):
+    B, H, S, D = 2, 2, 1024, 128
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=41, device=gpu)
+    mask = W.random_block_mask(S, 32, 0.5, seed=42, device=gpu, batch=B).clone()
+    mask[1, :, 77] = False  # a row that attends to nothing
+    me = mask.expand(B, H, S, S)
+    if route == "plain":
+        md = compute_mask_kernel(me, BQ, BK, pack_partial=False)
+    elif BQ == 256:
+        pytest.skip("no scheduled forward for BLOCK_Q = 256")
+    else:
+        md = compute_mask_kernel(me, BQ, BK, schedule="pairs" if route == "packed+pairs" else "persistent")
+    o, lse = sparse_attention(q, k, v, me, BQ, BK, mask_metadata=md, return_lse=True)
+    assert torch.equal(o, sparse_attention(q, k, v, me, BQ, BK, mask_metadata=md))
+    s = torch.einsum("bhqd,bhkd->bhqk", q.double(), k.double()) / math.sqrt(D)
+    want = torch.logsumexp(s.masked_fill(~me, -math.inf), dim=-1)
+    assert lse.shape == (B, H, S) and lse.dtype == torch.float32
+    assert (lse[1, :, 77] == -math.inf).all()
+    live = torch.isfinite(want)
+    assert torch.equal(live, torch.isfinite(lse))
+    # the row sum adds up P as rounded to bf16 for the P.V product: relative error of the sum below 2^-9
+    assert (lse[live].double() - want[live]).abs().max() <= 4e-3
