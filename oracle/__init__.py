@@ -226,3 +226,37 @@ def forward_dense_fp64(q, k, v, mask) -> np.ndarray:
     den = p.sum(axis=-1, keepdims=True)
     p = np.divide(p, den, out=np.zeros_like(p), where=den > 0)
     return np.einsum("bhqk,bhkd->bhqd", p, v)
+
+
+def backward_dense_fp64(q, k, v, mask, do):
+    """Gradients of :func:`forward_dense_fp64` with respect to q, k, v for the upstream gradient ``do``, in float64.
+
+    The reference has no backward pass (README.md:65 lists it as future work); this is the textbook derivative of
+    o = softmax(q kᵀ/√D + (mask ? 0 : −∞)) v, the function sparse_attn_kernel.py:149-185 computes:
+    P = softmax(S), dV = Pᵀ dO, dP = dO Vᵀ, dS = P ∘ (dP − rowsum(dO ∘ O)), dQ = dS K/√D, dK = dSᵀ Q/√D.
+    Rows with no attended key have P = 0 and contribute nothing.  Quadratic memory: small shapes only.
+    Returns (dq, dk, dv).
+    """
+    q = np.asarray(q, dtype=np.float64)
+    k = np.asarray(k, dtype=np.float64)
+    v = np.asarray(v, dtype=np.float64)
+    do = np.asarray(do, dtype=np.float64)
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    mask = np.broadcast_to(np.asarray(mask).astype(bool), (B, H, Sq, Sk))
+    scale = 1.0 / math.sqrt(D)
+    s = np.einsum("bhqd,bhkd->bhqk", q, k) * scale
+    s = np.where(mask, s, -np.inf)
+    mx = s.max(axis=-1, keepdims=True)
+    mx = np.where(np.isfinite(mx), mx, 0.0)
+    p = np.exp(s - mx)
+    den = p.sum(axis=-1, keepdims=True)
+    p = np.divide(p, den, out=np.zeros_like(p), where=den > 0)
+    o = np.einsum("bhqk,bhkd->bhqd", p, v)
+    dv = np.einsum("bhqk,bhqd->bhkd", p, do)
+    dp = np.einsum("bhqd,bhkd->bhqk", do, v)
+    delta = (do * o).sum(axis=-1, keepdims=True)
+    ds = p * (dp - delta)
+    dq = np.einsum("bhqk,bhkd->bhqd", ds, k) * scale
+    dk = np.einsum("bhqk,bhqd->bhkd", ds, q) * scale
+    return dq, dk, dv
