@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define SA_ABI_VERSION 6
+#define SA_ABI_VERSION 7
 
 enum sa_status {
     SA_OK = 0,
@@ -243,6 +243,37 @@ int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const 
                                const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int D, int BK,
                                int dtype, float sm_scale_log2, int num_splits, void *workspace, size_t workspace_bytes,
                                float *lse, const int64_t lse_strides[3], void *stream);
+
+/*
+ * Backward pass: dq, dk, dv from the upstream gradient d_o, for the function sa_sparse_attention_fwd computes
+ * (sparseattention/sparse_attn_kernel.py:149-185).  The reference has none ("Backwards pass + decode kernels",
+ * README.md:65); the derivative is the textbook one: P = exp(S - lse), dV = P^T dO, dP = dO V^T,
+ * dS = P o (dP - rowsum(dO o O)), dQ = scale dS K, dK = scale dS^T Q.
+ *
+ *   o, lse          outputs of sa_sparse_attention_fwd_lse for the same q, k, v, mask
+ *   q_* lists       sa_mask_classify of the mask with BQ = 128, BK = 64:  ids [B,H,Sq/128,Sk/64], lens [B,H,Sq/128]
+ *   k_* lists       sa_mask_classify of the TRANSPOSED mask (strides 2 and 3 swapped, Sq and Sk swapped) with
+ *                   BQ = 128, BK = 64:  ids [B,H,Sk/128,Sq/64], lens [B,H,Sk/128]
+ *   workspace       sa_bwd_workspace_bytes(B, H, Sq) bytes of device memory, 16-byte aligned
+ * D = 128, bf16 or fp16, Sq and Sk multiples of 128; tensors as for the forward (last dimension contiguous).
+ * The tile sizes of the backward are its own: they need not be those the forward ran with.
+ */
+size_t sa_bwd_workspace_bytes(int B, int H, int Sq);
+int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                            const void *v, const int64_t v_strides[4], const void *o, const int64_t o_strides[4],
+                            const void *d_o, const int64_t do_strides[4], const float *lse,
+                            const int64_t lse_strides[3], void *dq, const int64_t dq_strides[4], void *dk,
+                            const int64_t dk_strides[4], void *dv, const int64_t dv_strides[4], const uint8_t *mask,
+                            const int64_t mask_strides[4], const int32_t *q_full_ids,
+                            const int64_t q_full_ids_strides[4], const int32_t *q_full_lens,
+                            const int64_t q_full_lens_strides[3], const int32_t *q_part_ids,
+                            const int64_t q_part_ids_strides[4], const int32_t *q_part_lens,
+                            const int64_t q_part_lens_strides[3], const int32_t *k_full_ids,
+                            const int64_t k_full_ids_strides[4], const int32_t *k_full_lens,
+                            const int64_t k_full_lens_strides[3], const int32_t *k_part_ids,
+                            const int64_t k_part_ids_strides[4], const int32_t *k_part_lens,
+                            const int64_t k_part_lens_strides[3], void *workspace, size_t workspace_bytes, int B,
+                            int H, int Sq, int Sk, int D, int dtype, float sm_scale_log2, void *stream);
 
 #ifdef __cplusplus
 }

@@ -21,7 +21,7 @@ LIB_PATH = os.path.join(_HERE, "libsparseattn_hip.so")
 # mask source, so that the variants build in parallel.
 UNITS = [("sparseattn_api.hip", "sparseattn_api.o", []), ("mask_classify.hip", "mask_classify.o", []),
          ("fwd_schedule.hip", "fwd_schedule.o", []), ("sparse_fwd.hip", "sparse_fwd.o", []),
-         ("sparse_decode.hip", "sparse_decode.o", [])]
+         ("sparse_decode.hip", "sparse_decode.o", []), ("sparse_bwd.hip", "sparse_bwd.o", [])]
 UNITS += [("sparse_fwd_inst.hip", f"sparse_fwd_dt{dt}_pk{pk}_ps{ps}.o",
            [f"-DSA_FWD_DT={dt}", f"-DSA_FWD_PK={pk}", f"-DSA_FWD_PS={ps}"])
           for dt in (0, 1) for pk in (0, 1) for ps in (0, 1)]

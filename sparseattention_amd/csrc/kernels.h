@@ -109,4 +109,36 @@ struct DecodeParams {
 };
 hipError_t launch_decode(const DecodeParams &p, int dtype, int D, hipStream_t stream);
 
+// ---- backward ------------------------------------------------------------------------------------
+// One pass of the backward kernel (sparse_bwd.hip): tiles of 128 resident rows walk their lists of 64-row streamed
+// tiles.  dQ: resident q (x = q, g = dO), streamed keys (y = k, z = v), statistics per resident row.
+// dK / dV: resident keys (x = k, g = v), streamed queries (y = q, z = dO), statistics per streamed row, lists and
+// mask strides of the transposed mask.  D = 128.
+struct BwdParams {
+    const uint16_t *x, *g, *y, *z;
+    uint16_t *out;
+    int64_t xs[3], gs[3], ys[3], zs[3], outs[3];  // b, h, row strides in elements (d stride is 1)
+    const uint8_t *mask;
+    int64_t ms[2];     // mask strides along b and h in bytes
+    int64_t mrs, mcs;  // mask strides along the resident and the streamed rows in bytes
+    int mask_vec4;     // 1: mcs == 1 and 4-byte aligned rows
+    const int32_t *full_ids, *full_lens, *part_ids, *part_lens;  // per resident tile, streamed tiles of 64
+    int64_t fis[4], fls[3], pis[4], pls[3];
+    const float *stat_l, *stat_d;  // per query: lse / ln 2 (+inf for dead rows) and rowsum(dO o O)
+    int64_t sts[3];                // their b, h, row strides in elements (row stride 1 when queries are streamed)
+    int B, H, nR;                  // nR: resident tiles
+    float scale;                   // softmax scale / ln 2 (folded into x)
+    float out_scale;               // softmax scale for dQ and dK, 1 for dV
+};
+hipError_t launch_bwd(const BwdParams &p, int dtype, bool lane_stats, bool out_p, hipStream_t stream);
+
+struct BwdPrepParams {
+    const uint16_t *o, *d_o;
+    const float *lse;
+    int64_t os[3], dos[3], ls[3];
+    float *stat_l, *stat_d;  // [B*H*Sq] each, contiguous
+    int B, H, Sq;
+};
+hipError_t launch_bwd_prepare(const BwdPrepParams &p, int dtype, hipStream_t stream);
+
 }  // namespace sa

@@ -569,4 +569,163 @@ int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const 
     return SA_OK;
 }
 
+size_t sa_bwd_workspace_bytes(int B, int H, int Sq) {
+    if (B <= 0 || H <= 0 || Sq <= 0) return 0;
+    return (size_t)B * H * Sq * 2 * sizeof(float);
+}
+
+int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                            const void *v, const int64_t v_strides[4], const void *o, const int64_t o_strides[4],
+                            const void *d_o, const int64_t do_strides[4], const float *lse,
+                            const int64_t lse_strides[3], void *dq, const int64_t dq_strides[4], void *dk,
+                            const int64_t dk_strides[4], void *dv, const int64_t dv_strides[4], const uint8_t *mask,
+                            const int64_t mask_strides[4], const int32_t *q_full_ids,
+                            const int64_t q_full_ids_strides[4], const int32_t *q_full_lens,
+                            const int64_t q_full_lens_strides[3], const int32_t *q_part_ids,
+                            const int64_t q_part_ids_strides[4], const int32_t *q_part_lens,
+                            const int64_t q_part_lens_strides[3], const int32_t *k_full_ids,
+                            const int64_t k_full_ids_strides[4], const int32_t *k_full_lens,
+                            const int64_t k_full_lens_strides[3], const int32_t *k_part_ids,
+                            const int64_t k_part_ids_strides[4], const int32_t *k_part_lens,
+                            const int64_t k_part_lens_strides[3], void *workspace, size_t workspace_bytes, int B,
+                            int H, int Sq, int Sk, int D, int dtype, float sm_scale_log2, void *stream) {
+    g_error[0] = 0;
+    const void *ptrs[] = {q, k, v, o, d_o, lse, dq, dk, dv, mask, q_full_ids, q_full_lens, q_part_ids, q_part_lens,
+                          k_full_ids, k_full_lens, k_part_ids, k_part_lens, q_strides, k_strides, v_strides, o_strides,
+                          do_strides, lse_strides, dq_strides, dk_strides, dv_strides, mask_strides,
+                          q_full_ids_strides, q_full_lens_strides, q_part_ids_strides, q_part_lens_strides,
+                          k_full_ids_strides, k_full_lens_strides, k_part_ids_strides, k_part_lens_strides};
+    for (const void *ptr : ptrs)
+        if (!ptr) return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_bwd: null pointer argument");
+    if (const int rc = check_tiling(B, H, Sq, Sk, 128, 128)) return rc;  // tiles of 128 resident and 64 streamed rows both ways
+    if (D != 128) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_bwd: head dim %d (supported: 128)", D);
+    if (dtype != SA_DTYPE_BF16 && dtype != SA_DTYPE_FP16)
+        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_bwd: dtype code %d (supported: 0 = bf16, 1 = fp16)", dtype);
+    if (!(sm_scale_log2 > 0.f) || !(sm_scale_log2 < 3.0e38f))
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_bwd: sm_scale_log2 must be positive and finite");
+    if (Sq / 64 > 2048 || Sk / 64 > 2048)
+        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_bwd: more than 2048 tiles of 64 rows along Sq or Sk");
+    if ((int64_t)B * H > 65535) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_bwd: more than 65535 (b, h) planes");
+    const int64_t *st[9] = {q_strides, k_strides, v_strides, o_strides, do_strides, dq_strides, dk_strides, dv_strides};
+    const void *tp[8] = {q, k, v, o, d_o, dq, dk, dv};
+    const char *name[8] = {"q", "k", "v", "o", "do", "dq", "dk", "dv"};
+    for (int t = 0; t < 8; t++) {
+        if (st[t][3] != 1)
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_bwd: %s must be contiguous in its last dimension", name[t]);
+        if (!aligned(tp[t], 16) || st[t][0] % 8 || st[t][1] % 8 || st[t][2] % 8)
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_bwd: %s needs a 16-byte aligned base and strides that are multiples of 8 elements", name[t]);
+    }
+    for (int t = 5; t < 8; t++)
+        if (st[t][2] == 0 || (B > 1 && st[t][0] == 0) || (H > 1 && st[t][1] == 0))
+            return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_bwd: %s must not alias itself (zero stride)", name[t]);
+    const size_t need = sa_bwd_workspace_bytes(B, H, Sq);
+    if (!workspace || workspace_bytes < need || !aligned(workspace, 16))
+        return fail(SA_ERR_WORKSPACE, "sa_sparse_attention_bwd: 16-byte aligned workspace of %zu bytes required, %zu given", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    if (need / 2 >= (size_t)1 << 32) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_bwd: B*H*Sq too large");
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    const float sm_scale = sm_scale_log2 * 0.69314718056f;
+
+    // per query row: L = lse / ln 2 and Delta = rowsum(dO o O)
+    float *stat_l = static_cast<float *>(workspace);
+    float *stat_d = stat_l + (size_t)B * H * Sq;
+    sa::BwdPrepParams pp{};
+    pp.o = static_cast<const uint16_t *>(o);
+    pp.d_o = static_cast<const uint16_t *>(d_o);
+    pp.lse = lse;
+    for (int i = 0; i < 3; i++) {
+        pp.os[i] = o_strides[i];
+        pp.dos[i] = do_strides[i];
+        pp.ls[i] = lse_strides[i];
+    }
+    pp.stat_l = stat_l;
+    pp.stat_d = stat_d;
+    pp.B = B;
+    pp.H = H;
+    pp.Sq = Sq;
+    hipError_t e = sa::launch_bwd_prepare(pp, dtype, hs);
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_bwd: launch failed: %s", hipGetErrorString(e));
+
+    auto set3 = [](int64_t(&dst)[3], const int64_t *src) {
+        for (int i = 0; i < 3; i++) dst[i] = src[i];
+    };
+    sa::BwdParams bp{};
+    bp.mask = mask;
+    bp.ms[0] = mask_strides[0];
+    bp.ms[1] = mask_strides[1];
+    bp.stat_l = stat_l;
+    bp.stat_d = stat_d;
+    bp.sts[0] = (int64_t)H * Sq;
+    bp.sts[1] = Sq;
+    bp.sts[2] = 1;
+    bp.B = B;
+    bp.H = H;
+    bp.scale = sm_scale_log2;
+    const bool m4 = aligned(mask, 4) && mask_strides[0] % 4 == 0 && mask_strides[1] % 4 == 0;
+
+    // dQ: queries resident, keys streamed
+    bp.x = static_cast<const uint16_t *>(q);
+    bp.g = static_cast<const uint16_t *>(d_o);
+    bp.y = static_cast<const uint16_t *>(k);
+    bp.z = static_cast<const uint16_t *>(v);
+    bp.out = static_cast<uint16_t *>(dq);
+    set3(bp.xs, q_strides);
+    set3(bp.gs, do_strides);
+    set3(bp.ys, k_strides);
+    set3(bp.zs, v_strides);
+    set3(bp.outs, dq_strides);
+    bp.mrs = mask_strides[2];
+    bp.mcs = mask_strides[3];
+    bp.mask_vec4 = (m4 && bp.mcs == 1 && bp.mrs % 4 == 0) ? 1 : 0;
+    bp.full_ids = q_full_ids;
+    bp.full_lens = q_full_lens;
+    bp.part_ids = q_part_ids;
+    bp.part_lens = q_part_lens;
+    for (int i = 0; i < 4; i++) {
+        bp.fis[i] = q_full_ids_strides[i];
+        bp.pis[i] = q_part_ids_strides[i];
+    }
+    set3(bp.fls, q_full_lens_strides);
+    set3(bp.pls, q_part_lens_strides);
+    bp.nR = Sq / 128;
+    bp.out_scale = sm_scale;
+    e = sa::launch_bwd(bp, dtype, true, false, hs);
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_bwd: launch failed: %s", hipGetErrorString(e));
+
+    // dK and dV: keys resident, queries streamed; the mask is walked transposed
+    bp.x = static_cast<const uint16_t *>(k);
+    bp.g = static_cast<const uint16_t *>(v);
+    bp.y = static_cast<const uint16_t *>(q);
+    bp.z = static_cast<const uint16_t *>(d_o);
+    set3(bp.xs, k_strides);
+    set3(bp.gs, v_strides);
+    set3(bp.ys, q_strides);
+    set3(bp.zs, do_strides);
+    bp.mrs = mask_strides[3];
+    bp.mcs = mask_strides[2];
+    bp.mask_vec4 = (m4 && bp.mcs == 1 && bp.mrs % 4 == 0) ? 1 : 0;
+    bp.full_ids = k_full_ids;
+    bp.full_lens = k_full_lens;
+    bp.part_ids = k_part_ids;
+    bp.part_lens = k_part_lens;
+    for (int i = 0; i < 4; i++) {
+        bp.fis[i] = k_full_ids_strides[i];
+        bp.pis[i] = k_part_ids_strides[i];
+    }
+    set3(bp.fls, k_full_lens_strides);
+    set3(bp.pls, k_part_lens_strides);
+    bp.nR = Sk / 128;
+    bp.out = static_cast<uint16_t *>(dk);
+    set3(bp.outs, dk_strides);
+    bp.out_scale = sm_scale;
+    e = sa::launch_bwd(bp, dtype, false, false, hs);
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_bwd: launch failed: %s", hipGetErrorString(e));
+    bp.out = static_cast<uint16_t *>(dv);
+    set3(bp.outs, dv_strides);
+    bp.out_scale = 1.f;
+    e = sa::launch_bwd(bp, dtype, false, true, hs);
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_bwd: launch failed: %s", hipGetErrorString(e));
+    return SA_OK;
+}
+
 }  // extern "C"

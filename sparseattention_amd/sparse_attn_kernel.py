@@ -154,3 +154,86 @@ def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, m
             torch.cuda.current_stream(q.device).cuda_stream)
     _native.check(rc)
     return (o, lse) if return_lse else o
+
+
+class BackwardMetadata:
+    """Tile lists the backward pass walks: of the mask per 128 queries (KV tiles of 64 keys) and of the transposed
+    mask per 128 keys (tiles of 64 queries).  Built once per mask by :func:`compute_backward_metadata`."""
+
+    def __init__(self, by_query: MaskMetadata, by_key: MaskMetadata):
+        self.by_query = by_query
+        self.by_key = by_key
+
+
+def compute_backward_metadata(mask: torch.Tensor) -> BackwardMetadata:
+    """``mask``: bool [B,H,Sq,Sk] (broadcast views are fine), Sq and Sk multiples of 128."""
+    return BackwardMetadata(compute_mask_kernel(mask, 128, 64, pack_partial=False),
+                            compute_mask_kernel(mask.transpose(-1, -2), 128, 64, pack_partial=False))
+
+
+def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor,
+                              lse: torch.Tensor, mask: torch.Tensor, bwd_metadata: BackwardMetadata | None = None):
+    """Gradients (dq, dk, dv) of :func:`sparse_attention` for the upstream gradient ``do``.
+
+    The reference has no backward pass (README.md:65 lists it as future work); this differentiates its forward
+    (sparse_attn_kernel.py:149-185).  ``o`` and ``lse`` come from ``sparse_attention(..., return_lse=True)`` with the
+    same inputs.  D = 128, bf16/fp16, Sq and Sk multiples of 128.  The backward tiles the mask its own way
+    (128 x 64 both ways), whatever BLOCK_Q / BLOCK_K the forward used.
+    """
+    B, H, Sq, D = q.shape
+    Sk = k.shape[-2]
+    if not q.is_cuda:
+        raise RuntimeError("sparse_attention_backward needs its tensors on a ROCm GPU; there is no CPU path")
+    if q.dtype not in _DTYPES or any(t.dtype != q.dtype for t in (k, v, o, do)):
+        raise TypeError("q, k, v, o, do must share dtype bfloat16 or float16")
+    if lse.dtype != torch.float32 or tuple(lse.shape) != (B, H, Sq):
+        raise ValueError(f"lse: expected float32 {(B, H, Sq)}, got {lse.dtype} {tuple(lse.shape)}")
+    mask = mask.expand(B, H, Sq, Sk)
+    assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
+    if bwd_metadata is None:
+        bwd_metadata = compute_backward_metadata(mask)
+    sm_scale = D ** (-0.5) * 1 / math.log(2)
+    qc, kc, vc, oc, doc = (_kernel_ready(t) for t in (q, k, v, o, do))
+    dq, dk, dv = torch.empty_like(qc), torch.empty_like(kc), torch.empty_like(vc)
+    lib = _native.load()
+    S = _native.strides
+    lists = []
+    for md, shape in ((bwd_metadata.by_query, (B, H, Sq // 128, Sk // 64)), (bwd_metadata.by_key, (B, H, Sk // 128, Sq // 64))):
+        for t, shp in ((md.unmasked_kv_ids, shape), (md.unmasked_lens, shape[:3]), (md.masked_kv_ids, shape),
+                       (md.masked_lens, shape[:3])):
+            if tuple(t.shape) != shp or t.dtype != torch.int32 or t.device != q.device:
+                raise ValueError(f"bwd_metadata: expected int32 {shp} on {q.device}, got {t.dtype} {tuple(t.shape)}")
+            lists += [t.data_ptr(), S(t.stride())]
+    with torch.cuda.device(q.device):
+        ws_bytes = lib.sa_bwd_workspace_bytes(B, H, Sq)
+        ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=q.device)
+        rc = lib.sa_sparse_attention_bwd(
+            qc.data_ptr(), S(qc.stride()), kc.data_ptr(), S(kc.stride()), vc.data_ptr(), S(vc.stride()),
+            oc.data_ptr(), S(oc.stride()), doc.data_ptr(), S(doc.stride()), lse.data_ptr(), S(lse.stride()),
+            dq.data_ptr(), S(dq.stride()), dk.data_ptr(), S(dk.stride()), dv.data_ptr(), S(dv.stride()),
+            mask.data_ptr(), S(mask.stride()), *lists, ws.data_ptr(), ws_bytes,
+            B, H, Sq, Sk, D, _DTYPES[q.dtype], sm_scale, torch.cuda.current_stream(q.device).cuda_stream)
+    _native.check(rc)
+    return dq, dk, dv
+
+
+class _SparseAttentionFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, mask, BLOCK_Q, BLOCK_K, mask_metadata, bwd_metadata):
+        o, lse = sparse_attention(q, k, v, mask, BLOCK_Q, BLOCK_K, mask_metadata, return_lse=True)
+        ctx.save_for_backward(q, k, v, o, lse, mask)
+        ctx.bwd_metadata = bwd_metadata
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, o, lse, mask = ctx.saved_tensors
+        dq, dk, dv = sparse_attention_backward(do, q, k, v, o, lse, mask, ctx.bwd_metadata)
+        return dq, dk, dv, None, None, None, None, None
+
+
+def sparse_attention_trainable(q, k, v, mask, BLOCK_Q, BLOCK_K, mask_metadata: MaskMetadata | None = None,
+                               bwd_metadata: BackwardMetadata | None = None) -> torch.Tensor:
+    """:func:`sparse_attention` as a differentiable torch function (gradients for q, k, v through
+    :func:`sparse_attention_backward`)."""
+    return _SparseAttentionFunction.apply(q, k, v, mask, BLOCK_Q, BLOCK_K, mask_metadata, bwd_metadata)

@@ -1,0 +1,112 @@
+"""Parity of the backward pass (sa_sparse_attention_bwd through the Python binding).
+
+The reference has no backward; the checkers are the dense fp64 derivative of the oracle package (pinned against
+autograd and finite differences in tests/test_oracle_backward.py) on small shapes and torch autograd through
+fp32 masked SDPA on the same bf16 inputs on all shapes.  Tolerance: gradients of bf16 inputs within 2e-2 max-abs
+of the fp32 reference relative to the gradient's own scale (max-abs of the reference, at least 1)."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from sparseattention_amd import (compute_backward_metadata, compute_mask_kernel, sparse_attention,
+                                 sparse_attention_backward, sparse_attention_trainable, workloads as W)
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-2
+
+
+def sdpa_grads(q, k, v, mask, do):
+    q32, k32, v32 = (t.float().clone().requires_grad_(True) for t in (q, k, v))
+    o = F.scaled_dot_product_attention(q32, k32, v32, attn_mask=mask)
+    o.backward(do.float())
+    return q32.grad, k32.grad, v32.grad
+
+
+def check(got, want, what):
+    for g, w, name in zip(got, want, ("dq", "dk", "dv")):
+        assert not torch.isnan(g).any(), f"{what}: {name} has NaN"
+        scale = max(1.0, float(w.abs().max()))
+        err = float((g.float() - w.float().to(g.device)).abs().max()) / scale
+        assert err <= TOL, f"{what}: {name} off by {err:.3e} of its scale {scale:.2f}"
+
+
+def live_mask(S, block, p, seed, device, batch=None):
+    m = W.random_block_mask(S, block, p, seed=seed, device=device, batch=batch)
+    return m
+
+
+@pytest.mark.parametrize("S,block,p", [(256, 32, 0.3), (512, 64, 0.5), (512, 32, 0.7)])
+def test_against_oracle_and_autograd(gpu, S, block, p):
+    B, H, D = 1, 2, 128
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=S + block, device=gpu)
+    do = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(7)).to(gpu, torch.bfloat16)
+    mask = live_mask(S, block, p, seed=S, device=gpu)
+    o, lse = sparse_attention(q, k, v, mask, 128, 32, return_lse=True)
+    got = sparse_attention_backward(do, q, k, v, o, lse, mask)
+    torch.cuda.synchronize()
+    want = oracle.backward_dense_fp64(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(),
+                                      mask.cpu().numpy(), do.float().cpu().numpy())
+    check(got, [torch.from_numpy(w) for w in want], "vs oracle")
+    check(got, sdpa_grads(q, k, v, mask, do), "vs autograd")
+
+
+def test_causal_dense_and_cross_shapes(gpu):
+    B, H, D = 2, 2, 128
+    for Sq, Sk, kind in ((512, 512, "causal"), (256, 512, "dense"), (512, 256, "random")):
+        q, k, v = W.qkv(B, H, Sq, D, torch.bfloat16, seed=Sq + Sk, device=gpu, Sk=Sk)
+        do = torch.randn(B, H, Sq, D, generator=torch.Generator().manual_seed(8)).to(gpu, torch.bfloat16)
+        if kind == "causal":
+            mask = W.causal_mask(Sq, gpu)
+        elif kind == "dense":
+            mask = torch.ones(Sq, Sk, dtype=torch.bool, device=gpu)
+        else:
+            mask = (torch.rand(B, 1, Sq, Sk, generator=torch.Generator().manual_seed(9)) < 0.5).to(gpu)
+            mask[..., 0] = True
+        me = mask.expand(B, H, Sq, Sk)
+        o, lse = sparse_attention(q, k, v, me, 128, 64, return_lse=True)
+        got = sparse_attention_backward(do, q, k, v, o, lse, me)
+        check(got, sdpa_grads(q, k, v, mask, do), kind)
+
+
+def test_dead_rows_and_empty_tiles(gpu):
+    B, H, S, D = 1, 1, 512, 128
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=3, device=gpu)
+    do = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(4)).to(gpu, torch.bfloat16)
+    mask = live_mask(S, 64, 0.5, seed=5, device=gpu).clone()
+    mask[100] = False        # a query that attends to nothing
+    mask[:, 128:256] = False  # keys nobody attends to: dk = dv = 0 there
+    mask[0, 0] = True
+    o, lse = sparse_attention(q, k, v, mask, 128, 32, return_lse=True)
+    dq, dk, dv = sparse_attention_backward(do, q, k, v, o, lse, mask)
+    assert (dq[0, 0, 100] == 0).all() and (dk[0, 0, 128:256] == 0).all() and (dv[0, 0, 128:256] == 0).all()
+    want = oracle.backward_dense_fp64(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(),
+                                      mask.cpu().numpy(), do.float().cpu().numpy())
+    check((dq, dk, dv), [torch.from_numpy(w) for w in want], "dead rows")
+
+
+def test_autograd_function_and_metadata_reuse(gpu):
+    B, H, S, D = 1, 2, 256, 128
+    q, k, v = (t.requires_grad_(True) for t in W.qkv(B, H, S, D, torch.bfloat16, seed=11, device=gpu))
+    mask = W.causal_mask(S, gpu)
+    me = mask[None, None].expand(B, H, S, S)
+    md = compute_mask_kernel(me, 128, 32)
+    bmd = compute_backward_metadata(me)
+    o = sparse_attention_trainable(q, k, v, me, 128, 32, md, bmd)
+    do = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(12)).to(gpu, torch.bfloat16)
+    o.backward(do)
+    check((q.grad, k.grad, v.grad), sdpa_grads(q.detach(), k.detach(), v.detach(), mask, do), "autograd function")
+
+
+def test_fp16(gpu):
+    B, H, S, D = 1, 2, 256, 128
+    q, k, v = W.qkv(B, H, S, D, torch.float16, seed=13, device=gpu)
+    do = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(14)).to(gpu, torch.float16)
+    mask = live_mask(S, 32, 0.4, seed=15, device=gpu)
+    o, lse = sparse_attention(q, k, v, mask, 64, 32, return_lse=True)
+    got = sparse_attention_backward(do, q, k, v, o, lse, mask)
+    for g, w in zip(got, sdpa_grads(q, k, v, mask, do)):
+        assert float((g.float() - w).abs().max()) / max(1.0, float(w.abs().max())) <= 4e-3
