@@ -127,6 +127,7 @@ struct BwdParams {
     const float *stat_l, *stat_d;  // per query: lse / ln 2 (+inf for dead rows) and rowsum(dO o O)
     int64_t sts[3];                // their b, h, row strides in elements (row stride 1 when queries are streamed)
     int B, H, nR;                  // nR: resident tiles
+    int first_tile_first;          // launch order of a plane's tiles: 0 last tile first (queries), 1 first tile first (keys)
     float scale;                   // softmax scale / ln 2 (folded into x)
     float out_scale;               // softmax scale for dQ and dK, 1 for dV
 };

@@ -47,8 +47,19 @@ __global__ __launch_bounds__(256, 2) void sparse_bwd_kernel(const BwdParams p) {
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, hh = lane >> 5;
-    const int bh = blockIdx.y, b = bh / p.H, h = bh - b * p.H;
-    const int rt = p.nR - 1 - blockIdx.x;  // resident tile
+    // Workgroup -> (plane, resident tile) as in sparse_fwd_kernel: consecutive workgroup ids go to the 8 XCDs in turn,
+    // so each XCD gets a contiguous range of the plane-major order (the tiles that share K/V or Q/dO meet in one L2),
+    // planes two at a time with their tiles interleaved, the tile that is heaviest under causal-like masks first
+    // (the last queries, the first keys: p.first_tile_first).
+    const int total = gridDim.x, per = total >> 3;
+    int lin = blockIdx.x;
+    if (lin < (per << 3)) lin = (lin & 7) * per + (lin >> 3);
+    const int pair = lin / (2 * p.nR), pr = lin - pair * 2 * p.nR;
+    const bool paired = 2 * pair + 1 < p.B * p.H;
+    const int bh = 2 * pair + (paired ? (pr & 1) : 0);
+    const int order = paired ? (pr >> 1) : pr;
+    const int rt = p.first_tile_first ? order : p.nR - 1 - order;  // resident tile
+    const int b = bh / p.H, h = bh - b * p.H;
     const int rrow = rt * 128 + wave * 32 + l32;
 
     const uint16_t *ybase = p.y + b * p.ys[0] + h * p.ys[1];
@@ -291,7 +302,7 @@ hipError_t launch_bwd_one(const BwdParams &p, hipStream_t stream) {
     auto kern = sparse_bwd_kernel<DT, LANE_STATS, OUT_P>;
     static unsigned long long attr_done = 0;
     if (const hipError_t e0 = allow_dynamic_smem(kern, smem, attr_done); e0 != hipSuccess) return e0;
-    hipLaunchKernelGGL(kern, dim3(p.nR, p.B * p.H), dim3(256), smem, stream, p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)p.nR * (unsigned)p.B * (unsigned)p.H), dim3(256), smem, stream, p);
     return hipGetLastError();
 }
 

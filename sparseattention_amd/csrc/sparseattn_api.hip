@@ -605,7 +605,8 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
         return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_bwd: sm_scale_log2 must be positive and finite");
     if (Sq / 64 > 2048 || Sk / 64 > 2048)
         return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_bwd: more than 2048 tiles of 64 rows along Sq or Sk");
-    if ((int64_t)B * H > 65535) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_bwd: more than 65535 (b, h) planes");
+    if ((int64_t)B * H * ((Sq > Sk ? Sq : Sk) / 128) > 0x7fffffffLL)
+        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_bwd: more than 2^31-1 workgroups");
     const int64_t *st[9] = {q_strides, k_strides, v_strides, o_strides, do_strides, dq_strides, dk_strides, dv_strides};
     const void *tp[8] = {q, k, v, o, d_o, dq, dk, dv};
     const char *name[8] = {"q", "k", "v", "o", "do", "dq", "dk", "dv"};
@@ -688,6 +689,7 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
     set3(bp.fls, q_full_lens_strides);
     set3(bp.pls, q_part_lens_strides);
     bp.nR = Sq / 128;
+    bp.first_tile_first = 0;
     bp.out_scale = sm_scale;
     e = sa::launch_bwd(bp, dtype, true, false, hs);
     if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_bwd: launch failed: %s", hipGetErrorString(e));
@@ -715,6 +717,7 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
     set3(bp.fls, k_full_lens_strides);
     set3(bp.pls, k_part_lens_strides);
     bp.nR = Sk / 128;
+    bp.first_tile_first = 1;
     bp.out = static_cast<uint16_t *>(dk);
     set3(bp.outs, dk_strides);
     bp.out_scale = sm_scale;

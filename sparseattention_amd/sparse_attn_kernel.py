@@ -167,8 +167,14 @@ class BackwardMetadata:
 
 def compute_backward_metadata(mask: torch.Tensor) -> BackwardMetadata:
     """``mask``: bool [B,H,Sq,Sk] (broadcast views are fine), Sq and Sk multiples of 128."""
+    if mask.dim() != 4:
+        raise ValueError("mask must be [B,H,Sq,Sk] (broadcast views are fine)")
+    # the transposed mask as a tensor of its own, distinct planes only, so that its classification reads rows
+    B, H = mask.shape[:2]
+    distinct = mask[: 1 if mask.stride(0) == 0 else B, : 1 if mask.stride(1) == 0 else H]
+    transposed = distinct.transpose(-1, -2).contiguous().expand(B, H, mask.shape[3], mask.shape[2])
     return BackwardMetadata(compute_mask_kernel(mask, 128, 64, pack_partial=False),
-                            compute_mask_kernel(mask.transpose(-1, -2), 128, 64, pack_partial=False))
+                            compute_mask_kernel(transposed, 128, 64, pack_partial=False))
 
 
 def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor,
