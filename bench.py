@@ -17,6 +17,7 @@ the reference also excludes preprocessing from the forward time and reports it s
   across_p   the same forward on random block masks of sparsity p, a dense mask and the causal one
   variants   the headline workload through the other routes of the library (bool-mask reads, no schedule,
              persistent workgroups)
+  backward   dq, dk, dv of the headline workload (sparse_attention_backward) against the MFMA peak
   decode     the split-KV kernels for few query rows (sparse_attention_decode) against the HBM peak: K and V of
              the executed tiles are read once
   cpu_baseline / cpu_sdpa_baseline   the CPU oracle and torch's masked SDPA on a bounded sample
@@ -57,6 +58,7 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--no-classify", action="store_true", help="skip the mask-classification timing")
     ap.add_argument("--no-decode", action="store_true", help="skip the few-query-rows (decode) timing")
+    ap.add_argument("--no-backward", action="store_true", help="skip the backward-pass timing")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy a few times, so that a counter run over this command "
                          "holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -173,6 +175,38 @@ def classify_small_case(steps, warmup):
     _, full_ms = time_launches(lambda: compute_mask_kernel(me, BQ, BK, schedule="pairs"), steps, warmup)
     return {"workload": "compute_mask_kernel on the causal mask [4096,4096] = 16 MiB (latency bound)",
             "ms": round(ev_ms, 4), "with_pack_and_schedule_ms": round(full_ms, 4)}
+
+
+def backward_case(q, k, v, steps, warmup):
+    """dq, dk, dv of the headline workload (causal, B8 H32 S4096 D128 bf16); the backward tiles the mask 128 x 64
+    both ways.  Algorithmic work per executed tile: the five products of the derivative (S, dP, dQ, dK, dV) of
+    2*128*64*128 flop each; the three passes of the kernel recompute S twice and dP once, eight products in all."""
+    import torch
+    from sparseattention_amd import (compute_backward_metadata, compute_mask_kernel, sparse_attention,
+                                     sparse_attention_backward, workloads as W)
+
+    me = W.causal_mask(S, "cuda")[None, None].expand(B, H, S, S)
+    md = compute_mask_kernel(me, BQ, BK)
+    bmd = compute_backward_metadata(me)
+    o, lse = sparse_attention(q, k, v, me, BQ, BK, mask_metadata=md, return_lse=True)
+    do = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(3)).to("cuda", torch.bfloat16)
+    wall_ms, ev_ms = time_launches(lambda: sparse_attention_backward(do, q, k, v, o, lse, me, bmd), steps, warmup)
+    tq = int(bmd.by_query.unmasked_lens[0, 0].sum()) + int(bmd.by_query.masked_lens[0, 0].sum())
+    tk = int(bmd.by_key.unmasked_lens[0, 0].sum()) + int(bmd.by_key.masked_lens[0, 0].sum())
+    per_product = 2 * 128 * 64 * D
+    algorithmic = (3 * tq + 2 * tk) * per_product * B * H  # S, dP, dQ once per query-side tile; dK, dV per key-side tile
+    executed = (3 * tq + 5 * tk) * per_product * B * H
+    achieved = algorithmic / (ev_ms * 1e-3) / 1e12
+    return {
+        "workload": "dq, dk, dv of configs[1] (causal, B=8 H=32 S=4096 D=128 bf16), tiles 128x64 of the mask and of "
+                    "its transpose, o and lse from the forward, metadata precomputed",
+        "executed_tiles_per_plane": {"by_query": tq, "by_key": tk},
+        "ms": round(wall_ms, 4), "kernel_ms": round(ev_ms, 4),
+        "executed_tflops": round(executed / (ev_ms * 1e-3) / 1e12, 1),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "kernel": "sparse_bwd_kernel x3 (+ bwd_prepare_kernel)", "flop_per_launch": algorithmic},
+    }
 
 
 def decode_case(steps, warmup):
@@ -325,6 +359,8 @@ def main():
     if not args.no_classify:
         result["mask_classify"] = classify_case(max(10, args.steps // 2), max(3, args.warmup // 2))
         result["mask_classify_headline"] = classify_small_case(max(10, args.steps // 2), max(3, args.warmup // 2))
+    if not args.no_backward:
+        result["backward"] = backward_case(q, k, v, max(5, args.steps // 5), max(2, args.warmup // 3))
     del q, k, v
     if not args.no_decode:
         result["decode"] = decode_case(max(10, args.steps // 2), max(3, args.warmup // 2))

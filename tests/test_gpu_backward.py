@@ -110,3 +110,48 @@ def test_fp16(gpu):
     got = sparse_attention_backward(do, q, k, v, o, lse, mask)
     for g, w in zip(got, sdpa_grads(q, k, v, mask, do)):
         assert float((g.float() - w).abs().max()) / max(1.0, float(w.abs().max())) <= 4e-3
+
+
+def test_strided_storage_batch_masks_and_errors(gpu):
+    # [B,S,H,D] storage seen as [B,H,S,D]; one mask per batch element, broadcast over heads
+    B, H, S, D = 2, 3, 256, 128
+    g = torch.Generator().manual_seed(21)
+    q, k, v, do = (torch.randn(B, S, H, D, generator=g).to(gpu, torch.bfloat16).transpose(1, 2) for _ in range(4))
+    mask = live_mask(S, 32, 0.5, seed=22, device=gpu, batch=B)
+    me = mask.expand(B, H, S, S)
+    o, lse = sparse_attention(q, k, v, me, 128, 32, return_lse=True)
+    got = sparse_attention_backward(do, q, k, v, o, lse, me)
+    assert got[0].stride() == q.stride()
+    check(got, sdpa_grads(q, k, v, mask, do), "strided")
+    bmd = compute_backward_metadata(me)
+    assert bmd.by_key.unmasked_kv_ids.shape == (B, H, S // 128, S // 64) and bmd.by_key.unmasked_kv_ids.stride(1) == 0
+    again = sparse_attention_backward(do, q, k, v, o, lse, me, bmd)
+    assert all(torch.equal(a, b) for a, b in zip(got, again))
+    # head dim 64 and lengths that are not multiples of 128 have no backward kernel
+    from sparseattention_amd import _native
+    q64, k64, v64 = W.qkv(1, 1, 256, 64, torch.bfloat16, seed=23, device=gpu)
+    m64 = torch.ones(256, 256, dtype=torch.bool, device=gpu)
+    o64, lse64 = sparse_attention(q64, k64, v64, m64, 128, 32, return_lse=True)
+    with pytest.raises(_native.SparseAttnError):
+        sparse_attention_backward(o64, q64, k64, v64, o64, lse64, m64)
+    qs, ks, vs = W.qkv(1, 1, 192, 128, torch.bfloat16, seed=24, device=gpu)
+    ms = torch.ones(192, 192, dtype=torch.bool, device=gpu)
+    os_, lses = sparse_attention(qs, ks, vs, ms, 64, 32, return_lse=True)
+    with pytest.raises(AssertionError):  # the tiling asserts of compute_mask_kernel (mask_utils.py:89-90), 128 x 64 here
+        sparse_attention_backward(os_, qs, ks, vs, os_, lses, ms)
+
+
+def test_full_size_causal_planes_against_autograd(gpu):
+    B, H, S, D = 8, 32, 4096, 128
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=31, device=gpu)
+    do = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(32)).to(gpu, torch.bfloat16)
+    mask = W.causal_mask(S, gpu)
+    me = mask[None, None].expand(B, H, S, S)
+    o, lse = sparse_attention(q, k, v, me, 128, 32, return_lse=True)
+    dq, dk, dv = sparse_attention_backward(do, q, k, v, o, lse, me)
+    assert not (torch.isnan(dq).any() or torch.isnan(dk).any() or torch.isnan(dv).any())
+    for b, h in ((0, 0), (5, 13), (7, 31)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        check((dq[sl], dk[sl], dv[sl]), sdpa_grads(q[sl], k[sl], v[sl], mask, do[sl]), f"plane {b},{h}")
+    # every plane: dv is a P-weighted sum of dO rows, so column sums of dv equal those of dO (P rows sum to one)
+    assert (dv.float().sum(2) - do.float().sum(2)).abs().max() <= 0.5
