@@ -255,7 +255,7 @@ int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const 
  *   k_* lists       sa_mask_classify of the TRANSPOSED mask (strides 2 and 3 swapped, Sq and Sk swapped) with
  *                   BQ = 128, BK = 64:  ids [B,H,Sk/128,Sq/64], lens [B,H,Sk/128]
  *   workspace       sa_bwd_workspace_bytes(B, H, Sq) bytes of device memory, 16-byte aligned
- * D = 128, bf16 or fp16, Sq and Sk multiples of 128; tensors as for the forward (last dimension contiguous).
+ * D = 64 or 128, bf16 or fp16, Sq and Sk multiples of 128; tensors as for the forward (last dimension contiguous).
  * The tile sizes of the backward are its own: they need not be those the forward ran with.
  */
 size_t sa_bwd_workspace_bytes(int B, int H, int Sq);

@@ -113,7 +113,7 @@ hipError_t launch_decode(const DecodeParams &p, int dtype, int D, hipStream_t st
 // One pass of the backward kernel (sparse_bwd.hip): tiles of 128 resident rows walk their lists of 64-row streamed
 // tiles.  dQ: resident q (x = q, g = dO), streamed keys (y = k, z = v), statistics per resident row.
 // dK / dV: resident keys (x = k, g = v), streamed queries (y = q, z = dO), statistics per streamed row, lists and
-// mask strides of the transposed mask.  D = 128.
+// mask strides of the transposed mask.  D = 64 or 128.
 struct BwdParams {
     const uint16_t *x, *g, *y, *z;
     uint16_t *out;
@@ -131,7 +131,7 @@ struct BwdParams {
     float scale;                   // softmax scale / ln 2 (folded into x)
     float out_scale;               // softmax scale for dQ and dK, 1 for dV
 };
-hipError_t launch_bwd(const BwdParams &p, int dtype, bool lane_stats, bool out_p, hipStream_t stream);
+hipError_t launch_bwd(const BwdParams &p, int dtype, int D, bool lane_stats, bool out_p, hipStream_t stream);
 
 struct BwdPrepParams {
     const uint16_t *o, *d_o;
@@ -140,6 +140,6 @@ struct BwdPrepParams {
     float *stat_l, *stat_d;  // [B*H*Sq] each, contiguous
     int B, H, Sq;
 };
-hipError_t launch_bwd_prepare(const BwdPrepParams &p, int dtype, hipStream_t stream);
+hipError_t launch_bwd_prepare(const BwdPrepParams &p, int dtype, int D, hipStream_t stream);
 
 }  // namespace sa

@@ -25,20 +25,29 @@ namespace {
 
 constexpr int kBwdListCap = 2048;  // list entries kept in LDS (streamed length up to 131072)
 
-// XOR applied to the 16-byte piece index of LDS row `row` (D = 128: 16 pieces per row).  Bits 0-1 and 2-3 of the row
-// swapped: 16 consecutive rows get 16 different values (row-wise reads of one piece), and the 4 rows of a transposing
-// read get 4 different 64-byte groups.
-__device__ __forceinline__ int bwd_swizzle(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+// XOR applied to the 16-byte piece index of LDS row `row`.
+// D = 128 (16 pieces per row, rows 256 bytes apart): bits 0-1 and 2-3 of the row swapped.  16 consecutive rows get 16
+// different values (row-wise reads of one piece), and the 4 rows of a transposing read get 4 different 64-byte groups.
+// D = 64 (8 pieces, rows 128 bytes apart, so rows of equal parity share their banks): row bit 1 goes to bit 2, bits
+// 3 and 2 to bits 1 and 0.  The 8 rows of equal parity among 16 get 8 different values, and the two rows of equal
+// parity in a transposing read get different 64-byte groups.
+template <int D>
+__device__ __forceinline__ int bwd_swizzle(int row) {
+    if constexpr (D == 128) return ((row & 3) << 2) | ((row >> 2) & 3);
+    else return (((row >> 1) & 1) << 2) | (((row >> 3) & 1) << 1) | ((row >> 2) & 1);
+}
 
 // LANE_STATS: queries are the resident side (dQ).  OUT_P: the output product takes P and Z (dV) instead of dS and Y.
-template <int DT, bool LANE_STATS, bool OUT_P>
+template <int DT, int D, bool LANE_STATS, bool OUT_P>
 __global__ __launch_bounds__(256, 2) void sparse_bwd_kernel(const BwdParams p) {
     using E = Elem<DT>;
-    constexpr int D = 128;
+    static_assert(D == 128 || D == 64, "head dim");
     constexpr int ROWB = D * 2;
     constexpr int CBUF = 64 * ROWB;  // one streamed chunk of one tensor
     constexpr int NC = D / 16, NDB = D / 32;
-    constexpr int NLD = 4;           // direct loads per wave per chunk and tensor (4 rows each)
+    constexpr int PPR = ROWB / 16;   // 16-byte pieces per row
+    constexpr int RPI = 64 / PPR;    // rows per wave-wide direct load (1 KiB)
+    constexpr int NLD = 16 / RPI;    // direct loads per wave per chunk and tensor
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     // [Y stage 0,1][Z stage 0,1][stats stage 0,1: 64 L then 64 Delta floats][list]
     constexpr int STAT0 = 4 * CBUF;
@@ -105,7 +114,7 @@ __global__ __launch_bounds__(256, 2) void sparse_bwd_kernel(const BwdParams p) {
     // reads (rows 16kc + 4hh + j and + 8 of a 32-row block, 32-wide d block db), both through bwd_swizzle
     int noff[NC];
 #pragma unroll
-    for (int c = 0; c < NC; c++) noff[c] = l32 * ROWB + 16 * ((2 * c + hh) ^ bwd_swizzle(l32));
+    for (int c = 0; c < NC; c++) noff[c] = l32 * ROWB + 16 * ((2 * c + hh) ^ bwd_swizzle<D>(l32));
     int toff[2][NDB];
     {
         const int j = (lane & 15) >> 2;
@@ -114,19 +123,22 @@ __global__ __launch_bounds__(256, 2) void sparse_bwd_kernel(const BwdParams p) {
         for (int u = 0; u < 2; u++) {
             const int row = 4 * hh + j + 8 * u;
 #pragma unroll
-            for (int db = 0; db < NDB; db++)
-                toff[u][db] = row * ROWB + 64 * (db ^ j) + 16 * (x ^ ((hh + 2 * u) & 3)) + 8 * (lane & 1);
+            for (int db = 0; db < NDB; db++) {
+                // bwd_swizzle of row 16kc + 4hh + j + 8u, split into its 64-byte-group and its piece-in-group part
+                const int grp = D == 128 ? j : (j >> 1), pc = D == 128 ? ((hh + 2 * u) & 3) : ((u << 1) | hh);
+                toff[u][db] = row * ROWB + 64 * (db ^ grp) + 16 * (x ^ pc) + 8 * (lane & 1);
+            }
         }
     }
-    // direct loads: load i of this wave fills rows 4 (4i + wave) .. +3 of the chunk; the lane writes LDS piece
-    // lane % 16 of its row and therefore fetches the swizzled source piece
+    // direct loads: load i of this wave fills rows RPI (4i + wave) .. + RPI - 1 of the chunk; the lane writes LDS
+    // piece lane % PPR of its row and therefore fetches the swizzled source piece
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const SA_LDS uint8_t *)smem);
     uint32_t ld_yoff[NLD], ld_zoff[NLD];
 #pragma unroll
     for (int i = 0; i < NLD; i++) {
-        const int r = 4 * (4 * i + wave_u) + (lane >> 4);
-        const int piece = (lane & 15) ^ bwd_swizzle(r);
+        const int r = RPI * (4 * i + wave_u) + lane / PPR;
+        const int piece = (lane % PPR) ^ bwd_swizzle<D>(r);
         ld_yoff[i] = (uint32_t)((r * p.ys[2] + 8 * piece) * 2);
         ld_zoff[i] = (uint32_t)((r * p.zs[2] + 8 * piece) * 2);
     }
@@ -143,7 +155,7 @@ __global__ __launch_bounds__(256, 2) void sparse_bwd_kernel(const BwdParams p) {
         const int col = __builtin_amdgcn_readfirstlane(ent[t]);
 #pragma unroll
         for (int i = 0; i < NLD; i++) {
-            const uint32_t dst = 16 * (4 * i + wave_u) * 64;  // 4 rows of 256 bytes per load
+            const uint32_t dst = 1024 * (4 * i + wave_u);  // RPI rows per load
             dma16(ybase + (int64_t)col * p.ys[2], ld_yoff[i], lds0 + st * CBUF + dst);
             dma16(zbase + (int64_t)col * p.zs[2], ld_zoff[i], lds0 + (2 + st) * CBUF + dst);
         }
@@ -264,11 +276,12 @@ __global__ __launch_bounds__(256, 2) void sparse_bwd_kernel(const BwdParams p) {
 }
 
 // Per query row: Delta = sum_d dO o O, and L = lse / ln 2 (+inf for rows that attended to nothing, so that their
-// P = exp2(S - L) is 0).  16 lanes per row, 8 elements each (D = 128).
-template <int DT>
+// P = exp2(S - L) is 0).  D/8 lanes per row, 8 elements each.
+template <int DT, int D>
 __global__ __launch_bounds__(256) void bwd_prepare_kernel(const BwdPrepParams p) {
-    const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
-    const int part = threadIdx.x & 15;
+    constexpr int LPR = D / 8;  // lanes per row
+    const int64_t row = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
+    const int part = threadIdx.x % LPR;
     if (row >= (int64_t)p.B * p.H * p.Sq) return;
     const int q = (int)(row % p.Sq);
     const int bh = (int)(row / p.Sq);
@@ -278,17 +291,17 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(const BwdPrepParams p)
     float sum = 0.f;
 #pragma unroll
     for (int e = 0; e < 4; e++) {
+        const uint32_t ae = a[e], ge = g[e];  // (a bit cast applied to the vector element itself reads element 0)
         if constexpr (DT == 0) {
-            sum += __uint_as_float(a[e] << 16) * __uint_as_float(g[e] << 16);
-            sum += __uint_as_float(a[e] & 0xffff0000u) * __uint_as_float(g[e] & 0xffff0000u);
+            sum += __uint_as_float(ae << 16) * __uint_as_float(ge << 16);
+            sum += __uint_as_float(ae & 0xffff0000u) * __uint_as_float(ge & 0xffff0000u);
         } else {
-            const uint32_t ae = a[e], ge = g[e];  // (a bit cast applied to the vector element itself reads element 0)
             const f16x2 x = __builtin_bit_cast(f16x2, ae), y = __builtin_bit_cast(f16x2, ge);
             sum += (float)x.x * (float)y.x + (float)x.y * (float)y.y;
         }
     }
 #pragma unroll
-    for (int m = 8; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, 16);
+    for (int m = LPR / 2; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, LPR);
     if (part == 0) {
         const float lse = p.lse[b * p.ls[0] + h * p.ls[1] + (int64_t)q * p.ls[2]];
         p.stat_l[row] = lse == kNegInf ? __builtin_inff() : lse * 1.44269504089f;
@@ -296,37 +309,46 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(const BwdPrepParams p)
     }
 }
 
-template <int DT, bool LANE_STATS, bool OUT_P>
+template <int DT, int D, bool LANE_STATS, bool OUT_P>
 hipError_t launch_bwd_one(const BwdParams &p, hipStream_t stream) {
-    constexpr int smem = 4 * 64 * 256 + 2 * 512 + kBwdListCap * 4;
-    auto kern = sparse_bwd_kernel<DT, LANE_STATS, OUT_P>;
+    constexpr int smem = 4 * 64 * D * 2 + 2 * 512 + kBwdListCap * 4;
+    auto kern = sparse_bwd_kernel<DT, D, LANE_STATS, OUT_P>;
     static unsigned long long attr_done = 0;
     if (const hipError_t e0 = allow_dynamic_smem(kern, smem, attr_done); e0 != hipSuccess) return e0;
     hipLaunchKernelGGL(kern, dim3((unsigned)p.nR * (unsigned)p.B * (unsigned)p.H), dim3(256), smem, stream, p);
     return hipGetLastError();
 }
 
+template <int DT, int D>
+hipError_t launch_bwd_pass(const BwdParams &p, bool lane_stats, bool out_p, hipStream_t stream) {
+    if (lane_stats) return launch_bwd_one<DT, D, true, false>(p, stream);
+    return out_p ? launch_bwd_one<DT, D, false, true>(p, stream) : launch_bwd_one<DT, D, false, false>(p, stream);
+}
+
+template <int DT, int D>
+hipError_t launch_prepare_one(const BwdPrepParams &p, hipStream_t stream) {
+    const int64_t rows = (int64_t)p.B * p.H * p.Sq;
+    constexpr int RPB = 256 / (D / 8);  // rows per workgroup
+    hipLaunchKernelGGL((bwd_prepare_kernel<DT, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, stream, p);
+    return hipGetLastError();
+}
+
 }  // namespace
 
-hipError_t launch_bwd(const BwdParams &p, int dtype, bool lane_stats, bool out_p, hipStream_t stream) {
-    if (dtype == 0) {
-        if (lane_stats) return launch_bwd_one<0, true, false>(p, stream);
-        return out_p ? launch_bwd_one<0, false, true>(p, stream) : launch_bwd_one<0, false, false>(p, stream);
-    }
-    if (dtype == 1) {
-        if (lane_stats) return launch_bwd_one<1, true, false>(p, stream);
-        return out_p ? launch_bwd_one<1, false, true>(p, stream) : launch_bwd_one<1, false, false>(p, stream);
-    }
+hipError_t launch_bwd(const BwdParams &p, int dtype, int D, bool lane_stats, bool out_p, hipStream_t stream) {
+    if (dtype == 0 && D == 128) return launch_bwd_pass<0, 128>(p, lane_stats, out_p, stream);
+    if (dtype == 0 && D == 64) return launch_bwd_pass<0, 64>(p, lane_stats, out_p, stream);
+    if (dtype == 1 && D == 128) return launch_bwd_pass<1, 128>(p, lane_stats, out_p, stream);
+    if (dtype == 1 && D == 64) return launch_bwd_pass<1, 64>(p, lane_stats, out_p, stream);
     return hipErrorInvalidValue;
 }
 
-hipError_t launch_bwd_prepare(const BwdPrepParams &p, int dtype, hipStream_t stream) {
-    const int64_t rows = (int64_t)p.B * p.H * p.Sq;
-    const unsigned grid = (unsigned)((rows + 15) / 16);
-    if (dtype == 0) hipLaunchKernelGGL((bwd_prepare_kernel<0>), dim3(grid), dim3(256), 0, stream, p);
-    else if (dtype == 1) hipLaunchKernelGGL((bwd_prepare_kernel<1>), dim3(grid), dim3(256), 0, stream, p);
-    else return hipErrorInvalidValue;
-    return hipGetLastError();
+hipError_t launch_bwd_prepare(const BwdPrepParams &p, int dtype, int D, hipStream_t stream) {
+    if (dtype == 0 && D == 128) return launch_prepare_one<0, 128>(p, stream);
+    if (dtype == 0 && D == 64) return launch_prepare_one<0, 64>(p, stream);
+    if (dtype == 1 && D == 128) return launch_prepare_one<1, 128>(p, stream);
+    if (dtype == 1 && D == 64) return launch_prepare_one<1, 64>(p, stream);
+    return hipErrorInvalidValue;
 }
 
 }  // namespace sa

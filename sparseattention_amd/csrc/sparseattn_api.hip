@@ -598,7 +598,7 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
     for (const void *ptr : ptrs)
         if (!ptr) return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_bwd: null pointer argument");
     if (const int rc = check_tiling(B, H, Sq, Sk, 128, 128)) return rc;  // tiles of 128 resident and 64 streamed rows both ways
-    if (D != 128) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_bwd: head dim %d (supported: 128)", D);
+    if (D != 64 && D != 128) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_bwd: head dim %d (supported: 64, 128)", D);
     if (dtype != SA_DTYPE_BF16 && dtype != SA_DTYPE_FP16)
         return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_bwd: dtype code %d (supported: 0 = bf16, 1 = fp16)", dtype);
     if (!(sm_scale_log2 > 0.f) || !(sm_scale_log2 < 3.0e38f))
@@ -644,7 +644,7 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
     pp.B = B;
     pp.H = H;
     pp.Sq = Sq;
-    hipError_t e = sa::launch_bwd_prepare(pp, dtype, hs);
+    hipError_t e = sa::launch_bwd_prepare(pp, dtype, D, hs);
     if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_bwd: launch failed: %s", hipGetErrorString(e));
 
     auto set3 = [](int64_t(&dst)[3], const int64_t *src) {
@@ -691,7 +691,7 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
     bp.nR = Sq / 128;
     bp.first_tile_first = 0;
     bp.out_scale = sm_scale;
-    e = sa::launch_bwd(bp, dtype, true, false, hs);
+    e = sa::launch_bwd(bp, dtype, D, true, false, hs);
     if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_bwd: launch failed: %s", hipGetErrorString(e));
 
     // dK and dV: keys resident, queries streamed; the mask is walked transposed
@@ -721,12 +721,12 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
     bp.out = static_cast<uint16_t *>(dk);
     set3(bp.outs, dk_strides);
     bp.out_scale = sm_scale;
-    e = sa::launch_bwd(bp, dtype, false, false, hs);
+    e = sa::launch_bwd(bp, dtype, D, false, false, hs);
     if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_bwd: launch failed: %s", hipGetErrorString(e));
     bp.out = static_cast<uint16_t *>(dv);
     set3(bp.outs, dv_strides);
     bp.out_scale = 1.f;
-    e = sa::launch_bwd(bp, dtype, false, true, hs);
+    e = sa::launch_bwd(bp, dtype, D, false, true, hs);
     if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_bwd: launch failed: %s", hipGetErrorString(e));
     return SA_OK;
 }

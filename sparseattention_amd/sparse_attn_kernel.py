@@ -183,7 +183,7 @@ def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor
 
     The reference has no backward pass (README.md:65 lists it as future work); this differentiates its forward
     (sparse_attn_kernel.py:149-185).  ``o`` and ``lse`` come from ``sparse_attention(..., return_lse=True)`` with the
-    same inputs.  D = 128, bf16/fp16, Sq and Sk multiples of 128.  The backward tiles the mask its own way
+    same inputs.  D = 64 or 128, bf16/fp16, Sq and Sk multiples of 128.  The backward tiles the mask its own way
     (128 x 64 both ways), whatever BLOCK_Q / BLOCK_K the forward used.
     """
     B, H, Sq, D = q.shape
