@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define SA_ABI_VERSION 7
+#define SA_ABI_VERSION 8
 
 enum sa_status {
     SA_OK = 0,
@@ -254,6 +254,9 @@ int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const 
  *   q_* lists       sa_mask_classify of the mask with BQ = 128, BK = 64:  ids [B,H,Sq/128,Sk/64], lens [B,H,Sq/128]
  *   k_* lists       sa_mask_classify of the TRANSPOSED mask (strides 2 and 3 swapped, Sq and Sk swapped) with
  *                   BQ = 128, BK = 64:  ids [B,H,Sk/128,Sq/64], lens [B,H,Sk/128]
+ *   mask_t          optional: the transposed mask as a tensor [B,H,Sk,Sq] of its own (broadcast strides allowed), or
+ *                   NULL.  With it the dK and dV passes read the entries of PARTIAL tiles four at a time instead
+ *                   of byte-wise down the columns of `mask`.
  *   workspace       sa_bwd_workspace_bytes(B, H, Sq) bytes of device memory, 16-byte aligned
  * D = 64 or 128, bf16 or fp16, Sq and Sk multiples of 128; tensors as for the forward (last dimension contiguous).
  * The tile sizes of the backward are its own: they need not be those the forward ran with.
@@ -264,7 +267,8 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
                             const void *d_o, const int64_t do_strides[4], const float *lse,
                             const int64_t lse_strides[3], void *dq, const int64_t dq_strides[4], void *dk,
                             const int64_t dk_strides[4], void *dv, const int64_t dv_strides[4], const uint8_t *mask,
-                            const int64_t mask_strides[4], const int32_t *q_full_ids,
+                            const int64_t mask_strides[4], const uint8_t *mask_t, const int64_t mask_t_strides[4],
+                            const int32_t *q_full_ids,
                             const int64_t q_full_ids_strides[4], const int32_t *q_full_lens,
                             const int64_t q_full_lens_strides[3], const int32_t *q_part_ids,
                             const int64_t q_part_ids_strides[4], const int32_t *q_part_lens,

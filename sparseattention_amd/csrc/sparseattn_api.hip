@@ -579,7 +579,8 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
                             const void *d_o, const int64_t do_strides[4], const float *lse,
                             const int64_t lse_strides[3], void *dq, const int64_t dq_strides[4], void *dk,
                             const int64_t dk_strides[4], void *dv, const int64_t dv_strides[4], const uint8_t *mask,
-                            const int64_t mask_strides[4], const int32_t *q_full_ids,
+                            const int64_t mask_strides[4], const uint8_t *mask_t, const int64_t mask_t_strides[4],
+                            const int32_t *q_full_ids,
                             const int64_t q_full_ids_strides[4], const int32_t *q_full_lens,
                             const int64_t q_full_lens_strides[3], const int32_t *q_part_ids,
                             const int64_t q_part_ids_strides[4], const int32_t *q_part_lens,
@@ -694,7 +695,21 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
     e = sa::launch_bwd(bp, dtype, D, true, false, hs);
     if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_bwd: launch failed: %s", hipGetErrorString(e));
 
-    // dK and dV: keys resident, queries streamed; the mask is walked transposed
+    // dK and dV: keys resident, queries streamed; the mask is walked transposed, or read from the caller's
+    // transposed copy [B,H,Sk,Sq], whose rows are contiguous in the streamed direction
+    const uint8_t *mk = mask;
+    int64_t mk_b = mask_strides[0], mk_h = mask_strides[1], mk_r = mask_strides[3], mk_c = mask_strides[2];
+    if (mask_t) {
+        if (!mask_t_strides) return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_bwd: null pointer argument (mask_t_strides)");
+        mk = mask_t;
+        mk_b = mask_t_strides[0];
+        mk_h = mask_t_strides[1];
+        mk_r = mask_t_strides[2];
+        mk_c = mask_t_strides[3];
+    }
+    bp.mask = mk;
+    bp.ms[0] = mk_b;
+    bp.ms[1] = mk_h;
     bp.x = static_cast<const uint16_t *>(k);
     bp.g = static_cast<const uint16_t *>(v);
     bp.y = static_cast<const uint16_t *>(q);
@@ -703,9 +718,9 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
     set3(bp.gs, v_strides);
     set3(bp.ys, q_strides);
     set3(bp.zs, do_strides);
-    bp.mrs = mask_strides[3];
-    bp.mcs = mask_strides[2];
-    bp.mask_vec4 = (m4 && bp.mcs == 1 && bp.mrs % 4 == 0) ? 1 : 0;
+    bp.mrs = mk_r;
+    bp.mcs = mk_c;
+    bp.mask_vec4 = (aligned(mk, 4) && mk_b % 4 == 0 && mk_h % 4 == 0 && mk_c == 1 && mk_r % 4 == 0) ? 1 : 0;
     bp.full_ids = k_full_ids;
     bp.full_lens = k_full_lens;
     bp.part_ids = k_part_ids;

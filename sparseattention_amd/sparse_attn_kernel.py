@@ -160,9 +160,11 @@ class BackwardMetadata:
     """Tile lists the backward pass walks: of the mask per 128 queries (KV tiles of 64 keys) and of the transposed
     mask per 128 keys (tiles of 64 queries).  Built once per mask by :func:`compute_backward_metadata`."""
 
-    def __init__(self, by_query: MaskMetadata, by_key: MaskMetadata):
+    def __init__(self, by_query: MaskMetadata, by_key: MaskMetadata, transposed_mask: torch.Tensor | None = None):
         self.by_query = by_query
         self.by_key = by_key
+        #: bool [B,H,Sk,Sq], the mask transposed as a tensor of its own (distinct planes, expanded), or None
+        self.transposed_mask = transposed_mask
 
 
 def compute_backward_metadata(mask: torch.Tensor) -> BackwardMetadata:
@@ -174,7 +176,7 @@ def compute_backward_metadata(mask: torch.Tensor) -> BackwardMetadata:
     distinct = mask[: 1 if mask.stride(0) == 0 else B, : 1 if mask.stride(1) == 0 else H]
     transposed = distinct.transpose(-1, -2).contiguous().expand(B, H, mask.shape[3], mask.shape[2])
     return BackwardMetadata(compute_mask_kernel(mask, 128, 64, pack_partial=False),
-                            compute_mask_kernel(transposed, 128, 64, pack_partial=False))
+                            compute_mask_kernel(transposed, 128, 64, pack_partial=False), transposed)
 
 
 def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor,
@@ -210,6 +212,9 @@ def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor
             if tuple(t.shape) != shp or t.dtype != torch.int32 or t.device != q.device:
                 raise ValueError(f"bwd_metadata: expected int32 {shp} on {q.device}, got {t.dtype} {tuple(t.shape)}")
             lists += [t.data_ptr(), S(t.stride())]
+    mt = getattr(bwd_metadata, "transposed_mask", None)
+    if mt is not None and (tuple(mt.shape) != (B, H, Sk, Sq) or mt.dtype != torch.bool or mt.device != q.device):
+        raise ValueError(f"bwd_metadata.transposed_mask: expected bool {(B, H, Sk, Sq)} on {q.device}")
     with torch.cuda.device(q.device):
         ws_bytes = lib.sa_bwd_workspace_bytes(B, H, Sq)
         ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=q.device)
@@ -217,7 +222,9 @@ def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor
             qc.data_ptr(), S(qc.stride()), kc.data_ptr(), S(kc.stride()), vc.data_ptr(), S(vc.stride()),
             oc.data_ptr(), S(oc.stride()), doc.data_ptr(), S(doc.stride()), lse.data_ptr(), S(lse.stride()),
             dq.data_ptr(), S(dq.stride()), dk.data_ptr(), S(dk.stride()), dv.data_ptr(), S(dv.stride()),
-            mask.data_ptr(), S(mask.stride()), *lists, ws.data_ptr(), ws_bytes,
+            mask.data_ptr(), S(mask.stride()),
+            mt.data_ptr() if mt is not None else None, S(mt.stride()) if mt is not None else None,
+            *lists, ws.data_ptr(), ws_bytes,
             B, H, Sq, Sk, D, _DTYPES[q.dtype], sm_scale, torch.cuda.current_stream(q.device).cuda_stream)
     _native.check(rc)
     return dq, dk, dv

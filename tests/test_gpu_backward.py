@@ -152,3 +152,19 @@ def test_full_size_causal_planes_against_autograd(gpu):
         check((dq[sl], dk[sl], dv[sl]), sdpa_grads(q[sl], k[sl], v[sl], mask, do[sl]), f"plane {b},{h}")
     # every plane: dv is a P-weighted sum of dO rows, so column sums of dv equal those of dO (P rows sum to one)
     assert (dv.float().sum(2) - do.float().sum(2)).abs().max() <= 0.5
+
+
+def test_transposed_mask_copy_changes_nothing(gpu):
+    B, H, S, D = 2, 2, 512, 128
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=41, device=gpu)
+    do = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(42)).to(gpu, torch.bfloat16)
+    mask = (torch.rand(B, 1, S, S, generator=torch.Generator().manual_seed(43)) < 0.5).to(gpu)
+    me = mask.expand(B, H, S, S)
+    o, lse = sparse_attention(q, k, v, me, 128, 32, return_lse=True)
+    bmd = compute_backward_metadata(me)
+    assert bmd.transposed_mask.shape == (B, H, S, S) and bmd.transposed_mask.stride(1) == 0
+    with_copy = sparse_attention_backward(do, q, k, v, o, lse, me, bmd)
+    bmd.transposed_mask = None
+    without = sparse_attention_backward(do, q, k, v, o, lse, me, bmd)
+    assert all(torch.equal(a, b) for a, b in zip(with_copy, without))
+    check(with_copy, sdpa_grads(q, k, v, mask, do), "every tile partial")
