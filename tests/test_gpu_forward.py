@@ -306,5 +306,6 @@ def test_lse_output(gpu, route, BQ, BK):
     assert (lse[1, :, 77] == -math.inf).all()
     live = torch.isfinite(want)
     assert torch.equal(live, torch.isfinite(lse))
-    # the row sum adds up P as rounded to bf16 for the P.V product: relative error of the sum below 2^-9
-    assert (lse[live].double() - want[live]).abs().max() <= 4e-3
+    # the row sum adds up P as rounded to bf16 (8 significant bits) for the P.V product: a sum that one term
+    # dominates is off by up to 2^-8 of itself
+    assert (lse[live].double() - want[live]).abs().max() <= 6e-3
