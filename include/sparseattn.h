@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define SA_ABI_VERSION 8
+#define SA_ABI_VERSION 9
 
 enum sa_status {
     SA_OK = 0,
@@ -243,6 +243,18 @@ int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const 
                                const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int D, int BK,
                                int dtype, float sm_scale_log2, int num_splits, void *workspace, size_t workspace_bytes,
                                float *lse, const int64_t lse_strides[3], void *stream);
+
+/*
+ * Merge of n attention results over disjoint key ranges of the same queries (what sharding the key axis over
+ * devices, or over launches, ends with; the reference has no counterpart - it never hands out the row statistics):
+ *   o = sum_i exp(lse_i - lse) o_i,   lse = log sum_i exp(lse_i)     (rows with every lse_i = -inf give 0 and -inf)
+ * o_parts [n,B,H,Sq,D] and lse_parts [n,B,H,Sq] are outputs of sa_sparse_attention_fwd_lse (or of the decode entry)
+ * for the n key ranges; strides in elements, last dimension of o_parts and o contiguous.  lse may be NULL.
+ */
+int sa_merge_attention_parts(const void *o_parts, const int64_t o_parts_strides[5], const float *lse_parts,
+                             const int64_t lse_parts_strides[4], void *o, const int64_t o_strides[4], float *lse,
+                             const int64_t lse_strides[3], int n, int B, int H, int Sq, int D, int dtype,
+                             void *stream);
 
 /*
  * Backward pass: dq, dk, dv from the upstream gradient d_o, for the function sa_sparse_attention_fwd computes

@@ -12,9 +12,10 @@ The device work is done by hand-written gfx950 HIP kernels in ``libsparseattn_hi
 behind the C ABI of ``include/sparseattn.h``.
 """
 from .mask_utils import MaskMetadata, compute_mask_kernel, compute_mask_slow, select_block_sizes
-from .sparse_attn_kernel import (BackwardMetadata, compute_backward_metadata, sparse_attention,
-                                 sparse_attention_backward, sparse_attention_decode, sparse_attention_trainable)
+from .sparse_attn_kernel import (BackwardMetadata, compute_backward_metadata, merge_attention_parts, sparse_attention,
+                                 sparse_attention_backward, sparse_attention_decode, sparse_attention_kv_split,
+                                 sparse_attention_trainable)
 
 __all__ = ["MaskMetadata", "compute_mask_kernel", "compute_mask_slow", "select_block_sizes", "sparse_attention",
            "sparse_attention_decode", "sparse_attention_backward", "sparse_attention_trainable", "BackwardMetadata",
-           "compute_backward_metadata"]
+           "compute_backward_metadata", "merge_attention_parts", "sparse_attention_kv_split"]

@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsparseattn_hip.so")
 
-SA_ABI_VERSION = 8
+SA_ABI_VERSION = 9
 SA_OK = 0
 SA_ERR_INVALID_ARGUMENT = -1
 SA_ERR_UNSUPPORTED = -2
@@ -39,6 +39,7 @@ EXPORTS = (
     "sa_decode_num_splits",
     "sa_decode_workspace_bytes",
     "sa_sparse_attention_decode",
+    "sa_merge_attention_parts",
     "sa_bwd_workspace_bytes",
     "sa_sparse_attention_bwd",
 )
@@ -109,6 +110,8 @@ def load() -> ctypes.CDLL:
         [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [ctypes.c_int] * 7 + [ctypes.c_float, ctypes.c_int]
         + [_vp, ctypes.c_size_t] + [_vp, _i64p] + [_vp]
     )
+    lib.sa_merge_attention_parts.restype = ctypes.c_int
+    lib.sa_merge_attention_parts.argtypes = [_vp, _i64p] * 4 + [ctypes.c_int] * 6 + [_vp]
     lib.sa_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.sa_bwd_workspace_bytes.argtypes = [ctypes.c_int] * 3
     lib.sa_sparse_attention_bwd.restype = ctypes.c_int

@@ -109,6 +109,18 @@ struct DecodeParams {
 };
 hipError_t launch_decode(const DecodeParams &p, int dtype, int D, hipStream_t stream);
 
+// Merge of n attention results computed over disjoint key ranges (outputs and row log-sum-exps).
+struct MergeParams {
+    const uint16_t *o_parts;  // [n,B,H,Sq,D]
+    const float *lse_parts;   // [n,B,H,Sq]
+    uint16_t *o;
+    float *lse;               // optional
+    int64_t ops[4], lps[4];   // part, b, h, row strides in elements (d stride is 1)
+    int64_t os[3], lses[3];
+    int n, B, H, Sq, D;
+};
+hipError_t launch_merge_parts(const MergeParams &p, int dtype, hipStream_t stream);
+
 // ---- backward ------------------------------------------------------------------------------------
 // One pass of the backward kernel (sparse_bwd.hip): tiles of 128 resident rows walk their lists of 64-row streamed
 // tiles.  dQ: resident q (x = q, g = dO), streamed keys (y = k, z = v), statistics per resident row.

@@ -314,6 +314,53 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(const DecodeParams p)
     for (int j = 0; j < NV; j += 2) *(uint32_t *)(orow + j) = E::pack2(out[j] * inv, out[j + 1] * inv);
 }
 
+// Merge of n attention results over disjoint key ranges: o = sum_i exp(lse_i - lse) o_i, lse = log sum_i exp(lse_i).
+// One thread per 8 output elements.
+template <int DT>
+__global__ __launch_bounds__(256) void merge_parts_kernel(const MergeParams p) {
+    using E = Elem<DT>;
+    const int per_row = p.D / 8;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t row = idx / per_row;
+    const int part = (int)(idx - row * per_row);
+    if (row >= (int64_t)p.B * p.H * p.Sq) return;
+    const int q = (int)(row % p.Sq);
+    const int bh = (int)(row / p.Sq);
+    const int b = bh / p.H, h = bh - b * p.H;
+    const float *lp = p.lse_parts + b * p.lps[1] + h * p.lps[2] + (int64_t)q * p.lps[3];
+    float M = kNegInf;
+    for (int i = 0; i < p.n; i++) M = fmaxf(M, lp[i * p.lps[0]]);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float L = 0.f;
+    if (M != kNegInf) {
+        for (int i = 0; i < p.n; i++) {
+            const float w = __expf(lp[i * p.lps[0]] - M);  // 0 for parts whose keys this row does not attend to
+            L += w;
+            const u32x4 x = *(const u32x4 *)(p.o_parts + i * p.ops[0] + b * p.ops[1] + h * p.ops[2] +
+                                             (int64_t)q * p.ops[3] + 8 * part);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const uint32_t xe = x[e];
+                if constexpr (DT == 0) {
+                    acc[2 * e] += w * __uint_as_float(xe << 16);
+                    acc[2 * e + 1] += w * __uint_as_float(xe & 0xffff0000u);
+                } else {
+                    const f16x2 hx = __builtin_bit_cast(f16x2, xe);
+                    acc[2 * e] += w * (float)hx.x;
+                    acc[2 * e + 1] += w * (float)hx.y;
+                }
+            }
+        }
+    }
+    const float inv = L > 0.f ? 1.f / L : 0.f;
+    u32x4 out;
+#pragma unroll
+    for (int e = 0; e < 4; e++) out[e] = E::pack2(acc[2 * e] * inv, acc[2 * e + 1] * inv);
+    *(u32x4 *)(p.o + b * p.os[0] + h * p.os[1] + (int64_t)q * p.os[2] + 8 * part) = out;
+    if (p.lse != nullptr && part == 0)
+        p.lse[b * p.lses[0] + h * p.lses[1] + (int64_t)q * p.lses[2]] = L > 0.f ? M + __logf(L) : kNegInf;
+}
+
 template <int DT, int D>
 hipError_t launch_decode_one(const DecodeParams &p, hipStream_t stream) {
     constexpr int smem = decode_smem_bytes<D>();
@@ -328,6 +375,15 @@ hipError_t launch_decode_one(const DecodeParams &p, hipStream_t stream) {
 }
 
 }  // namespace
+
+hipError_t launch_merge_parts(const MergeParams &p, int dtype, hipStream_t stream) {
+    const int64_t threads = (int64_t)p.B * p.H * p.Sq * (p.D / 8);
+    const unsigned grid = (unsigned)((threads + 255) / 256);
+    if (dtype == 0) hipLaunchKernelGGL((merge_parts_kernel<0>), dim3(grid), dim3(256), 0, stream, p);
+    else if (dtype == 1) hipLaunchKernelGGL((merge_parts_kernel<1>), dim3(grid), dim3(256), 0, stream, p);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
 
 hipError_t launch_decode(const DecodeParams &p, int dtype, int D, hipStream_t stream) {
     if (dtype == 0 && D == 128) return launch_decode_one<0, 128>(p, stream);

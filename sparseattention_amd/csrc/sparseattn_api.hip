@@ -746,4 +746,47 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
     return SA_OK;
 }
 
+int sa_merge_attention_parts(const void *o_parts, const int64_t o_parts_strides[5], const float *lse_parts,
+                             const int64_t lse_parts_strides[4], void *o, const int64_t o_strides[4], float *lse,
+                             const int64_t lse_strides[3], int n, int B, int H, int Sq, int D, int dtype,
+                             void *stream) {
+    g_error[0] = 0;
+    if (!o_parts || !o_parts_strides || !lse_parts || !lse_parts_strides || !o || !o_strides)
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_merge_attention_parts: null pointer argument");
+    if (n <= 0 || B <= 0 || H <= 0 || Sq <= 0 || D <= 0)
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_merge_attention_parts: n, B, H, Sq, D must be positive");
+    if (D % 8) return fail(SA_ERR_UNSUPPORTED, "sa_merge_attention_parts: D %d (supported: multiples of 8)", D);
+    if (dtype != SA_DTYPE_BF16 && dtype != SA_DTYPE_FP16)
+        return fail(SA_ERR_UNSUPPORTED, "sa_merge_attention_parts: dtype code %d (supported: 0 = bf16, 1 = fp16)", dtype);
+    if (o_parts_strides[4] != 1 || o_strides[3] != 1)
+        return fail(SA_ERR_UNSUPPORTED, "sa_merge_attention_parts: o_parts and o must be contiguous in their last dimension");
+    if (!aligned(o_parts, 16) || !aligned(o, 16) || o_parts_strides[0] % 8 || o_parts_strides[1] % 8 ||
+        o_parts_strides[2] % 8 || o_parts_strides[3] % 8 || o_strides[0] % 8 || o_strides[1] % 8 || o_strides[2] % 8)
+        return fail(SA_ERR_UNSUPPORTED, "sa_merge_attention_parts: o_parts and o need 16-byte aligned bases and strides that are multiples of 8 elements");
+    if (lse && !lse_strides) return fail(SA_ERR_INVALID_ARGUMENT, "sa_merge_attention_parts: null pointer argument (lse_strides)");
+    if ((int64_t)B * H * Sq * (D / 8) / 256 > 0x7fffffffLL)
+        return fail(SA_ERR_UNSUPPORTED, "sa_merge_attention_parts: more than 2^31-1 workgroups");
+    sa::MergeParams mp{};
+    mp.o_parts = static_cast<const uint16_t *>(o_parts);
+    mp.lse_parts = lse_parts;
+    mp.o = static_cast<uint16_t *>(o);
+    mp.lse = lse;
+    for (int i = 0; i < 4; i++) {
+        mp.ops[i] = o_parts_strides[i];
+        mp.lps[i] = lse_parts_strides[i];
+    }
+    for (int i = 0; i < 3; i++) {
+        mp.os[i] = o_strides[i];
+        mp.lses[i] = lse ? lse_strides[i] : 0;
+    }
+    mp.n = n;
+    mp.B = B;
+    mp.H = H;
+    mp.Sq = Sq;
+    mp.D = D;
+    const hipError_t e = sa::launch_merge_parts(mp, dtype, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_merge_attention_parts: launch failed: %s", hipGetErrorString(e));
+    return SA_OK;
+}
+
 }  // extern "C"

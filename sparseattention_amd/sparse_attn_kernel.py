@@ -250,3 +250,48 @@ def sparse_attention_trainable(q, k, v, mask, BLOCK_Q, BLOCK_K, mask_metadata: M
     """:func:`sparse_attention` as a differentiable torch function (gradients for q, k, v through
     :func:`sparse_attention_backward`)."""
     return _SparseAttentionFunction.apply(q, k, v, mask, BLOCK_Q, BLOCK_K, mask_metadata, bwd_metadata)
+
+
+def merge_attention_parts(o_parts: torch.Tensor, lse_parts: torch.Tensor, return_lse: bool = False):
+    """Merge attention results computed over disjoint key ranges of the same queries.
+
+    ``o_parts`` [n,B,H,Sq,D] (bf16/fp16) and ``lse_parts`` [n,B,H,Sq] (float32) as returned, per key range, by
+    ``sparse_attention(..., return_lse=True)``: ``o = Σ_i exp(lse_i − lse) o_i`` with ``lse = logsumexp_i lse_i``.
+    This is the exchange a key-axis sharding of the forward ends with (no counterpart in the reference).
+    """
+    if o_parts.dim() != 5 or lse_parts.shape != o_parts.shape[:4] or lse_parts.dtype != torch.float32:
+        raise ValueError("o_parts must be [n,B,H,Sq,D] and lse_parts float32 [n,B,H,Sq]")
+    if o_parts.dtype not in _DTYPES or not o_parts.is_cuda:
+        raise TypeError("o_parts must be a bfloat16 or float16 tensor on a ROCm GPU")
+    n, B, H, Sq, D = o_parts.shape
+    if o_parts.stride(-1) != 1 or o_parts.data_ptr() % 16 or any(s % 8 for s in o_parts.stride()[:-1]):
+        o_parts = o_parts.contiguous()
+    o = torch.empty(B, H, Sq, D, dtype=o_parts.dtype, device=o_parts.device)
+    lse = torch.empty(B, H, Sq, dtype=torch.float32, device=o_parts.device) if return_lse else None
+    S = _native.strides
+    with torch.cuda.device(o_parts.device):
+        rc = _native.load().sa_merge_attention_parts(
+            o_parts.data_ptr(), S(o_parts.stride()), lse_parts.data_ptr(), S(lse_parts.stride()),
+            o.data_ptr(), S(o.stride()), lse.data_ptr() if return_lse else None, S(lse.stride()) if return_lse else None,
+            n, B, H, Sq, D, _DTYPES[o_parts.dtype], torch.cuda.current_stream(o_parts.device).cuda_stream)
+    _native.check(rc)
+    return (o, lse) if return_lse else o
+
+
+def sparse_attention_kv_split(q, k, v, mask, BLOCK_Q, BLOCK_K, num_splits: int, return_lse: bool = False):
+    """:func:`sparse_attention` with the key axis cut into ``num_splits`` equal ranges, each run as a forward of
+    its own (own tile lists) and merged by :func:`merge_attention_parts`: what one device per range would do.
+    Useful on one device when there are too few Q tiles to fill it (a few hundred query rows against long keys)."""
+    B, H, Sq, D = q.shape
+    Sk = k.shape[-2]
+    if Sk % (num_splits * BLOCK_K):
+        raise ValueError(f"Sk ({Sk}) must be a multiple of num_splits * BLOCK_K ({num_splits} * {BLOCK_K})")
+    mask = mask.expand(B, H, Sq, Sk)
+    step = Sk // num_splits
+    o_parts = torch.empty(num_splits, B, H, Sq, D, dtype=q.dtype, device=q.device)
+    lse_parts = torch.empty(num_splits, B, H, Sq, dtype=torch.float32, device=q.device)
+    for i in range(num_splits):
+        sl = slice(i * step, (i + 1) * step)
+        o_parts[i], lse_parts[i] = sparse_attention(q, k[:, :, sl], v[:, :, sl], mask[..., sl], BLOCK_Q, BLOCK_K,
+                                                    return_lse=True)
+    return merge_attention_parts(o_parts, lse_parts, return_lse)
