@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define SA_ABI_VERSION 9
+#define SA_ABI_VERSION 10
 
 enum sa_status {
     SA_OK = 0,
@@ -269,6 +269,10 @@ int sa_merge_attention_parts(const void *o_parts, const int64_t o_parts_strides[
  *   mask_t          optional: the transposed mask as a tensor [B,H,Sk,Sq] of its own (broadcast strides allowed), or
  *                   NULL.  With it the dK and dV passes read the entries of PARTIAL tiles four at a time instead
  *                   of byte-wise down the columns of `mask`.
+ *   q_packed, k_packed   optional: outputs of sa_mask_pack_partial for the two tilings above (the mask with BQ = 128,
+ *                   BK = 64 and the q_* lists; the transposed mask with BQ = 128, BK = 64 and the k_* lists), or
+ *                   NULL.  A pass that has its packed buffer reads no mask; with both, `mask` and `mask_t` may be
+ *                   NULL, so the bool tensors can be released after preprocessing.
  *   workspace       sa_bwd_workspace_bytes(B, H, Sq) bytes of device memory, 16-byte aligned
  * D = 64 or 128, bf16 or fp16, Sq and Sk multiples of 128; tensors as for the forward (last dimension contiguous).
  * The tile sizes of the backward are its own: they need not be those the forward ran with.
@@ -280,7 +284,8 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
                             const int64_t lse_strides[3], void *dq, const int64_t dq_strides[4], void *dk,
                             const int64_t dk_strides[4], void *dv, const int64_t dv_strides[4], const uint8_t *mask,
                             const int64_t mask_strides[4], const uint8_t *mask_t, const int64_t mask_t_strides[4],
-                            const int32_t *q_full_ids,
+                            const uint8_t *q_packed, const int64_t q_packed_strides[2], const uint8_t *k_packed,
+                            const int64_t k_packed_strides[2], const int32_t *q_full_ids,
                             const int64_t q_full_ids_strides[4], const int32_t *q_full_lens,
                             const int64_t q_full_lens_strides[3], const int32_t *q_part_ids,
                             const int64_t q_part_ids_strides[4], const int32_t *q_part_lens,

@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsparseattn_hip.so")
 
-SA_ABI_VERSION = 9
+SA_ABI_VERSION = 10
 SA_OK = 0
 SA_ERR_INVALID_ARGUMENT = -1
 SA_ERR_UNSUPPORTED = -2
@@ -116,7 +116,7 @@ def load() -> ctypes.CDLL:
     lib.sa_bwd_workspace_bytes.argtypes = [ctypes.c_int] * 3
     lib.sa_sparse_attention_bwd.restype = ctypes.c_int
     lib.sa_sparse_attention_bwd.argtypes = (
-        [_vp, _i64p] * 11 + [_vp, _i64p] * 8 + [_vp, ctypes.c_size_t] + [ctypes.c_int] * 6 + [ctypes.c_float, _vp]
+        [_vp, _i64p] * 13 + [_vp, _i64p] * 8 + [_vp, ctypes.c_size_t] + [ctypes.c_int] * 6 + [ctypes.c_float, _vp]
     )
     if lib.sa_abi_version() != SA_ABI_VERSION:
         raise RuntimeError(f"libsparseattn_hip ABI {lib.sa_abi_version()} != expected {SA_ABI_VERSION}")

@@ -134,6 +134,10 @@ struct BwdParams {
     int64_t ms[2];     // mask strides along b and h in bytes
     int64_t mrs, mcs;  // mask strides along the resident and the streamed rows in bytes
     int mask_vec4;     // 1: mcs == 1 and 4-byte aligned rows
+    // Bit-packed PARTIAL tiles of this pass's tiling (PackParams layout, tiles of 128 x 64), or null: then `mask`.
+    const uint8_t *packed;
+    int64_t pks[2];    // bytes between packed planes along b and h
+    int nS;            // streamed tiles per resident tile (slots in `packed`)
     const int32_t *full_ids, *full_lens, *part_ids, *part_lens;  // per resident tile, streamed tiles of 64
     int64_t fis[4], fls[3], pis[4], pls[3];
     const float *stat_l, *stat_d;  // per query: lse / ln 2 (+inf for dead rows) and rowsum(dO o O)

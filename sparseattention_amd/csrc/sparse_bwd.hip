@@ -78,6 +78,8 @@ __global__ __launch_bounds__(256, 2) void sparse_bwd_kernel(const BwdParams p) {
     const int F = p.full_lens[b * p.fls[0] + h * p.fls[1] + rt * p.fls[2]];
     const int T = F + p.part_lens[b * p.pls[0] + h * p.pls[1] + rt * p.pls[2]];  // chunks = list entries
     const uint8_t *mrow = p.mask + b * p.ms[0] + h * p.ms[1] + (int64_t)rrow * p.mrs;
+    // this lane's row in a packed tile: 8 bytes per row, 1024 per tile, nS tiles per resident tile
+    const uint8_t *prow = p.packed + b * p.pks[0] + h * p.pks[1] + (int64_t)rt * p.nS * 1024 + (wave * 32 + l32) * 8;
     const float *statL = p.stat_l + b * p.sts[0] + h * p.sts[1];
     const float *statD = p.stat_d + b * p.sts[0] + h * p.sts[1];
     // bytes from a query's L to its Delta (both live in one workspace, less than 4 GiB apart)
@@ -165,7 +167,13 @@ __global__ __launch_bounds__(256, 2) void sparse_bwd_kernel(const BwdParams p) {
                 dma16(statL + col, off, lds0 + STAT0 + st * 512);
             }
         }
-        if (t >= F) {
+        if (t >= F && p.packed != nullptr) {  // the row's 64 bits of the tile in slot t - F
+            const u32x2 w = *(const u32x2 *)(prow + (int64_t)(t - F) * 1024);
+            mk[0] = w.x;
+            mk[1] = w.y;
+#pragma unroll
+            for (int i = 2; i < 8; i++) mk[i] = 0u;
+        } else if (t >= F) {
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
@@ -199,11 +207,24 @@ __global__ __launch_bounds__(256, 2) void sparse_bwd_kernel(const BwdParams p) {
                 for (int c = 0; c < NC; c++) dp = E::mfma(*(const u32x4 *)(zb + 32 * kb * ROWB + noff[c]), gf[c], dp);
             }
             if (t >= F) {
+                // w: bit 8g + jj says whether this lane's entry (streamed row 32kb + 8g + 4hh + jj) attends
+                uint32_t w;
+                if (p.packed != nullptr) {  // bit k of the packed word: streamed row 32kb + k
+                    w = mk[kb] >> (4 * hh);
+                } else {  // one byte per entry: the non-zero bytes of each dword become four bits
+                    w = 0u;
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const uint32_t m = mk[4 * kb + g];
+                        const uint32_t nz = ((((m & 0x7f7f7f7fu) + 0x7f7f7f7fu) | m) >> 7) & 0x01010101u;
+                        w |= ((nz * 0x01020408u) >> 24) << (8 * g);
+                    }
+                }
 #pragma unroll
                 for (int g = 0; g < 4; g++)
 #pragma unroll
                     for (int jj = 0; jj < 4; jj++)
-                        if (((mk[4 * kb + g] >> (8 * jj)) & 0xffu) == 0u) s[4 * g + jj] = kNegInf;
+                        if (((w >> (8 * g + jj)) & 1u) == 0u) s[4 * g + jj] = kNegInf;
             }
             // P^T = exp2(S^T - L) and, unless OUT_P, dS^T = P^T o (dP^T - Delta); rounded to the input type
             uint32_t pw[8];

@@ -580,7 +580,8 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
                             const int64_t lse_strides[3], void *dq, const int64_t dq_strides[4], void *dk,
                             const int64_t dk_strides[4], void *dv, const int64_t dv_strides[4], const uint8_t *mask,
                             const int64_t mask_strides[4], const uint8_t *mask_t, const int64_t mask_t_strides[4],
-                            const int32_t *q_full_ids,
+                            const uint8_t *q_packed, const int64_t q_packed_strides[2], const uint8_t *k_packed,
+                            const int64_t k_packed_strides[2], const int32_t *q_full_ids,
                             const int64_t q_full_ids_strides[4], const int32_t *q_full_lens,
                             const int64_t q_full_lens_strides[3], const int32_t *q_part_ids,
                             const int64_t q_part_ids_strides[4], const int32_t *q_part_lens,
@@ -591,9 +592,13 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
                             const int64_t k_part_lens_strides[3], void *workspace, size_t workspace_bytes, int B,
                             int H, int Sq, int Sk, int D, int dtype, float sm_scale_log2, void *stream) {
     g_error[0] = 0;
-    const void *ptrs[] = {q, k, v, o, d_o, lse, dq, dk, dv, mask, q_full_ids, q_full_lens, q_part_ids, q_part_lens,
+    if (!mask && !(q_packed && k_packed))
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_bwd: null pointer argument (mask, without both packed buffers)");
+    if ((q_packed && !q_packed_strides) || (k_packed && !k_packed_strides))
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_bwd: null pointer argument (packed strides)");
+    const void *ptrs[] = {q, k, v, o, d_o, lse, dq, dk, dv, q_full_ids, q_full_lens, q_part_ids, q_part_lens,
                           k_full_ids, k_full_lens, k_part_ids, k_part_lens, q_strides, k_strides, v_strides, o_strides,
-                          do_strides, lse_strides, dq_strides, dk_strides, dv_strides, mask_strides,
+                          do_strides, lse_strides, dq_strides, dk_strides, dv_strides,
                           q_full_ids_strides, q_full_lens_strides, q_part_ids_strides, q_part_lens_strides,
                           k_full_ids_strides, k_full_lens_strides, k_part_ids_strides, k_part_lens_strides};
     for (const void *ptr : ptrs)
@@ -651,6 +656,14 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
     auto set3 = [](int64_t(&dst)[3], const int64_t *src) {
         for (int i = 0; i < 3; i++) dst[i] = src[i];
     };
+    if (mask && !mask_strides) return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_bwd: null pointer argument (mask_strides)");
+    const uint8_t *pk[2] = {q_packed, k_packed};
+    const int64_t *pks[2] = {q_packed_strides, k_packed_strides};
+    for (int i = 0; i < 2; i++)
+        if (pk[i] && (!aligned(pk[i], 8) || (B > 1 && pks[i][0] % 8) || (H > 1 && pks[i][1] % 8)))
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_bwd: packed buffers need 8-byte aligned bases and plane strides");
+    const int64_t no_strides[4] = {0, 0, 0, 0};
+    if (!mask) mask_strides = no_strides;
     sa::BwdParams bp{};
     bp.mask = mask;
     bp.ms[0] = mask_strides[0];
@@ -663,7 +676,7 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
     bp.B = B;
     bp.H = H;
     bp.scale = sm_scale_log2;
-    const bool m4 = aligned(mask, 4) && mask_strides[0] % 4 == 0 && mask_strides[1] % 4 == 0;
+    const bool m4 = mask && aligned(mask, 4) && mask_strides[0] % 4 == 0 && mask_strides[1] % 4 == 0;
 
     // dQ: queries resident, keys streamed
     bp.x = static_cast<const uint16_t *>(q);
@@ -689,6 +702,10 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
     }
     set3(bp.fls, q_full_lens_strides);
     set3(bp.pls, q_part_lens_strides);
+    bp.packed = q_packed;
+    bp.pks[0] = q_packed ? q_packed_strides[0] : 0;
+    bp.pks[1] = q_packed ? q_packed_strides[1] : 0;
+    bp.nS = Sk / 64;
     bp.nR = Sq / 128;
     bp.first_tile_first = 0;
     bp.out_scale = sm_scale;
@@ -731,6 +748,10 @@ int sa_sparse_attention_bwd(const void *q, const int64_t q_strides[4], const voi
     }
     set3(bp.fls, k_full_lens_strides);
     set3(bp.pls, k_part_lens_strides);
+    bp.packed = k_packed;
+    bp.pks[0] = k_packed ? k_packed_strides[0] : 0;
+    bp.pks[1] = k_packed ? k_packed_strides[1] : 0;
+    bp.nS = Sq / 64;
     bp.nR = Sk / 128;
     bp.first_tile_first = 1;
     bp.out = static_cast<uint16_t *>(dk);

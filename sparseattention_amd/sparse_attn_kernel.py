@@ -158,7 +158,10 @@ def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, m
 
 class BackwardMetadata:
     """Tile lists the backward pass walks: of the mask per 128 queries (KV tiles of 64 keys) and of the transposed
-    mask per 128 keys (tiles of 64 queries).  Built once per mask by :func:`compute_backward_metadata`."""
+    mask per 128 keys (tiles of 64 queries).  Built once per mask by :func:`compute_backward_metadata`.
+
+    When both lists carry ``packed_masks`` (the PARTIAL tiles at one bit per entry), the backward reads those and
+    neither the mask nor its transposed copy, so both bool tensors can be released after this preprocessing."""
 
     def __init__(self, by_query: MaskMetadata, by_key: MaskMetadata, transposed_mask: torch.Tensor | None = None):
         self.by_query = by_query
@@ -167,26 +170,32 @@ class BackwardMetadata:
         self.transposed_mask = transposed_mask
 
 
-def compute_backward_metadata(mask: torch.Tensor) -> BackwardMetadata:
-    """``mask``: bool [B,H,Sq,Sk] (broadcast views are fine), Sq and Sk multiples of 128."""
+def compute_backward_metadata(mask: torch.Tensor, pack_partial: bool = True) -> BackwardMetadata:
+    """``mask``: bool [B,H,Sq,Sk] (broadcast views are fine), Sq and Sk multiples of 128.
+
+    ``pack_partial``: bit-pack the PARTIAL tiles of both tilings (2 * Sq*Sk/8 bytes per distinct plane at most) and
+    drop the transposed copy; otherwise keep that copy (Sq*Sk bytes per distinct plane) for the key passes."""
     if mask.dim() != 4:
         raise ValueError("mask must be [B,H,Sq,Sk] (broadcast views are fine)")
     # the transposed mask as a tensor of its own, distinct planes only, so that its classification reads rows
     B, H = mask.shape[:2]
     distinct = mask[: 1 if mask.stride(0) == 0 else B, : 1 if mask.stride(1) == 0 else H]
     transposed = distinct.transpose(-1, -2).contiguous().expand(B, H, mask.shape[3], mask.shape[2])
-    return BackwardMetadata(compute_mask_kernel(mask, 128, 64, pack_partial=False),
-                            compute_mask_kernel(transposed, 128, 64, pack_partial=False), transposed)
+    return BackwardMetadata(compute_mask_kernel(mask, 128, 64, pack_partial=pack_partial),
+                            compute_mask_kernel(transposed, 128, 64, pack_partial=pack_partial),
+                            None if pack_partial else transposed)
 
 
 def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor,
-                              lse: torch.Tensor, mask: torch.Tensor, bwd_metadata: BackwardMetadata | None = None):
+                              lse: torch.Tensor, mask: torch.Tensor | None,
+                              bwd_metadata: BackwardMetadata | None = None):
     """Gradients (dq, dk, dv) of :func:`sparse_attention` for the upstream gradient ``do``.
 
     The reference has no backward pass (README.md:65 lists it as future work); this differentiates its forward
     (sparse_attn_kernel.py:149-185).  ``o`` and ``lse`` come from ``sparse_attention(..., return_lse=True)`` with the
     same inputs.  D = 64 or 128, bf16/fp16, Sq and Sk multiples of 128.  The backward tiles the mask its own way
-    (128 x 64 both ways), whatever BLOCK_Q / BLOCK_K the forward used.
+    (128 x 64 both ways), whatever BLOCK_Q / BLOCK_K the forward used.  ``mask`` may be None when ``bwd_metadata``
+    carries the packed PARTIAL tiles of both tilings.
     """
     B, H, Sq, D = q.shape
     Sk = k.shape[-2]
@@ -196,22 +205,35 @@ def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor
         raise TypeError("q, k, v, o, do must share dtype bfloat16 or float16")
     if lse.dtype != torch.float32 or tuple(lse.shape) != (B, H, Sq):
         raise ValueError(f"lse: expected float32 {(B, H, Sq)}, got {lse.dtype} {tuple(lse.shape)}")
-    mask = mask.expand(B, H, Sq, Sk)
-    assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
+    if mask is not None:
+        mask = mask.expand(B, H, Sq, Sk)
+        assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
+        if mask.device != q.device:
+            raise ValueError("mask must be on the same device as q")
     if bwd_metadata is None:
+        if mask is None:
+            raise ValueError("sparse_attention_backward needs the mask or a BackwardMetadata with packed tiles")
         bwd_metadata = compute_backward_metadata(mask)
     sm_scale = D ** (-0.5) * 1 / math.log(2)
     qc, kc, vc, oc, doc = (_kernel_ready(t) for t in (q, k, v, o, do))
     dq, dk, dv = torch.empty_like(qc), torch.empty_like(kc), torch.empty_like(vc)
     lib = _native.load()
     S = _native.strides
-    lists = []
+    lists, packs = [], []
     for md, shape in ((bwd_metadata.by_query, (B, H, Sq // 128, Sk // 64)), (bwd_metadata.by_key, (B, H, Sk // 128, Sq // 64))):
         for t, shp in ((md.unmasked_kv_ids, shape), (md.unmasked_lens, shape[:3]), (md.masked_kv_ids, shape),
                        (md.masked_lens, shape[:3])):
             if tuple(t.shape) != shp or t.dtype != torch.int32 or t.device != q.device:
                 raise ValueError(f"bwd_metadata: expected int32 {shp} on {q.device}, got {t.dtype} {tuple(t.shape)}")
             lists += [t.data_ptr(), S(t.stride())]
+        pk = getattr(md, "packed_masks", None)
+        if pk is not None and (tuple(pk.shape) != shape + (1024,) or pk.dtype != torch.uint8 or pk.device != q.device
+                               or pk.stride()[2:] != (shape[3] * 1024, 1024, 1)):
+            raise ValueError(f"bwd_metadata packed_masks: expected uint8 {shape + (1024,)} on {q.device} with "
+                             f"contiguous tiles, got {pk.dtype} {tuple(pk.shape)} strides {pk.stride()}")
+        packs += [pk.data_ptr(), S(pk.stride()[:2])] if pk is not None else [None, None]
+    if mask is None and None in packs:
+        raise ValueError("sparse_attention_backward without a mask needs packed_masks in both lists of bwd_metadata")
     mt = getattr(bwd_metadata, "transposed_mask", None)
     if mt is not None and (tuple(mt.shape) != (B, H, Sk, Sq) or mt.dtype != torch.bool or mt.device != q.device):
         raise ValueError(f"bwd_metadata.transposed_mask: expected bool {(B, H, Sk, Sq)} on {q.device}")
@@ -222,9 +244,9 @@ def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor
             qc.data_ptr(), S(qc.stride()), kc.data_ptr(), S(kc.stride()), vc.data_ptr(), S(vc.stride()),
             oc.data_ptr(), S(oc.stride()), doc.data_ptr(), S(doc.stride()), lse.data_ptr(), S(lse.stride()),
             dq.data_ptr(), S(dq.stride()), dk.data_ptr(), S(dk.stride()), dv.data_ptr(), S(dv.stride()),
-            mask.data_ptr(), S(mask.stride()),
+            mask.data_ptr() if mask is not None else None, S(mask.stride()) if mask is not None else None,
             mt.data_ptr() if mt is not None else None, S(mt.stride()) if mt is not None else None,
-            *lists, ws.data_ptr(), ws_bytes,
+            *packs, *lists, ws.data_ptr(), ws_bytes,
             B, H, Sq, Sk, D, _DTYPES[q.dtype], sm_scale, torch.cuda.current_stream(q.device).cuda_stream)
     _native.check(rc)
     return dq, dk, dv

@@ -161,10 +161,51 @@ def test_transposed_mask_copy_changes_nothing(gpu):
     mask = (torch.rand(B, 1, S, S, generator=torch.Generator().manual_seed(43)) < 0.5).to(gpu)
     me = mask.expand(B, H, S, S)
     o, lse = sparse_attention(q, k, v, me, 128, 32, return_lse=True)
-    bmd = compute_backward_metadata(me)
+    bmd = compute_backward_metadata(me, pack_partial=False)
+    assert bmd.by_query.packed_masks is None and bmd.by_key.packed_masks is None
     assert bmd.transposed_mask.shape == (B, H, S, S) and bmd.transposed_mask.stride(1) == 0
     with_copy = sparse_attention_backward(do, q, k, v, o, lse, me, bmd)
     bmd.transposed_mask = None
     without = sparse_attention_backward(do, q, k, v, o, lse, me, bmd)
     assert all(torch.equal(a, b) for a, b in zip(with_copy, without))
     check(with_copy, sdpa_grads(q, k, v, mask, do), "every tile partial")
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_packed_partial_tiles_replace_both_masks(gpu, D, dtype):
+    # the same gradients, bit for bit, from the packed PARTIAL tiles as from the bool mask and its transposed copy;
+    # with packed tiles in both lists no mask is passed at all
+    B, H, Sq, Sk = 2, 3, 384, 640
+    q, _, _ = W.qkv(B, H, Sq, D, dtype, seed=51, device=gpu)
+    _, k, v = W.qkv(B, H, Sk, D, dtype, seed=52, device=gpu)
+    do = torch.randn(B, H, Sq, D, generator=torch.Generator().manual_seed(53)).to(gpu, dtype)
+    g = torch.Generator().manual_seed(54)
+    # squares of 128 in turn full, ragged and empty, so both tilings (128 x 64 each way) see all three kinds; the
+    # ragged ones mix random entries with empty blocks of 32; one mask per batch element
+    i, j = torch.arange(Sq // 128)[:, None], torch.arange(Sk // 128)[None, :]
+    kind = ((i + 2 * j) % 3).repeat_interleave(128, 0).repeat_interleave(128, 1)
+    fine = torch.rand(B, 1, Sq, Sk, generator=g) < 0.6
+    holes = (torch.rand(B, 1, Sq // 32, Sk // 32, generator=g) < 0.3).repeat_interleave(32, 2).repeat_interleave(32, 3)
+    mask = ((kind == 0) | ((kind == 1) & fine & ~holes)).to(gpu)
+    mask[..., 0] = True
+    me = mask.expand(B, H, Sq, Sk)
+    o, lse = sparse_attention(q, k, v, me, 128, 32, return_lse=True)
+    plain = compute_backward_metadata(me, pack_partial=False)
+    packed = compute_backward_metadata(me)
+    assert packed.transposed_mask is None
+    assert packed.by_query.packed_masks.shape == (B, H, Sq // 128, Sk // 64, 1024)
+    assert packed.by_key.packed_masks.shape == (B, H, Sk // 128, Sq // 64, 1024)
+    assert packed.by_key.packed_masks.stride(1) == 0
+    assert int(packed.by_query.masked_lens.sum()) > 0 and int(packed.by_query.unmasked_lens.sum()) > 0
+    want = sparse_attention_backward(do, q, k, v, o, lse, me, plain)
+    got = sparse_attention_backward(do, q, k, v, o, lse, None, packed)
+    assert all(torch.equal(a, b) for a, b in zip(got, want))
+    # one orientation packed, the other from the mask
+    packed.by_key.packed_masks = None
+    mixed = sparse_attention_backward(do, q, k, v, o, lse, me, packed)
+    assert all(torch.equal(a, b) for a, b in zip(mixed, want))
+    with pytest.raises(ValueError):
+        sparse_attention_backward(do, q, k, v, o, lse, None, packed)
+    if dtype == torch.bfloat16:
+        check(got, sdpa_grads(q, k, v, mask, do), "packed tiles")
