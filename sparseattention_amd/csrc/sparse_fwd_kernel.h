@@ -365,11 +365,17 @@ __global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(co
         if constexpr (MODE != 2) {
             const int j = kEntryByLoad ? ((RPI * NW * i) >> LBKC) : (rbase >> LBKC);
 #pragma unroll
-            for (int jj = 1; jj < EPC; jj++)
+            for (int jj = 1; jj < EPC; jj++) {
+                const uint16_t *kc = pl.kp[jj], *vc = pl.vp[jj];
+                // With more than two candidates and an entry that depends on the wave, the compiler would turn
+                // this chain into one load at a variable index, which keeps the plan in scratch memory; values
+                // that passed through an (empty) asm statement are no loads any more.
+                if constexpr (!kEntryByLoad && EPC > 2) asm volatile("" : "+s"(kc), "+s"(vc));
                 if (j == jj) {
-                    ks_ = pl.kp[jj];
-                    vs_ = pl.vp[jj];
+                    ks_ = kc;
+                    vs_ = vc;
                 }
+            }
         }
         if ((piece & 1) == 0) dma16(ks_, ld_koff[i], lds0 + buf * KBUF + rbase * ROWB);
         else dma16(vs_, ld_voff[i], lds0 + NS * KBUF + buf * VBUF + rbase * ROWB);
