@@ -165,6 +165,24 @@ def classify_case(steps, warmup):
     }
 
 
+def terms_case(steps, warmup):
+    """The same composed mask from its formula: lists and packed PARTIAL tiles without the 1 GiB tensor."""
+    import torch
+    from sparseattention_amd import block_term, causal_term, compute_mask_terms
+
+    Sbig = 32768
+    terms = [causal_term(window=1024), block_term((0, 2048), (0, 2048))]
+    md = compute_mask_terms(terms, 1, 32, Sbig, Sbig, BQ, BK, device="cuda")
+    full, part = int(md.unmasked_lens[0, 0].sum()), int(md.masked_lens[0, 0].sum())
+    _, ev_ms = time_launches(lambda: compute_mask_terms(terms, 1, 32, Sbig, Sbig, BQ, BK, device="cuda"), steps, warmup)
+    return {
+        "workload": "compute_mask_terms on (k<=q and q-k<1024) or (q<2048 and k<2048), S=32768, tiles 128x32: "
+                    "classification from the formula, lists, packed PARTIAL tiles; no mask tensor",
+        "full_tiles": full, "partial_tiles": part, "ms": round(ev_ms, 4),
+        "entries_per_s": round(Sbig * Sbig / (ev_ms * 1e-3), 1),
+    }
+
+
 def classify_small_case(steps, warmup):
     """Preprocessing of the headline mask itself ([4096,4096] = 16 MiB): launch-latency bound."""
     import torch
@@ -358,6 +376,7 @@ def main():
         result["across_p"] = [{kk: vv for kk, vv in r.items() if not kk.startswith("_")} for r in rows]
     if not args.no_classify:
         result["mask_classify"] = classify_case(max(10, args.steps // 2), max(3, args.warmup // 2))
+        result["mask_terms"] = terms_case(max(10, args.steps // 2), max(3, args.warmup // 2))
         result["mask_classify_headline"] = classify_small_case(max(10, args.steps // 2), max(3, args.warmup // 2))
     if not args.no_backward:
         result["backward"] = backward_case(q, k, v, max(5, args.steps // 5), max(2, args.warmup // 3))

@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define SA_ABI_VERSION 10
+#define SA_ABI_VERSION 11
 
 enum sa_status {
     SA_OK = 0,
@@ -52,6 +52,16 @@ enum sa_dtype {
     SA_DTYPE_BF16 = 0,
     SA_DTYPE_FP16 = 1
 };
+
+/* Conditions of one term of a mask given by a formula (sa_mask_classify_terms). */
+enum sa_term_flags {
+    SA_TERM_BACK = 1,     /* (q + offset) - k < back                                   */
+    SA_TERM_AHEAD = 2,    /* k - (q + offset) < ahead        (ahead = 1: causal)       */
+    SA_TERM_Q_RANGE = 4,  /* q_lo <= q < q_hi                                          */
+    SA_TERM_K_RANGE = 8,  /* k_lo <= k < k_hi                                          */
+    SA_TERM_SAME_DOC = 16 /* doc_q[b][q] == doc_k[b][k]                                */
+};
+#define SA_MAX_MASK_TERMS 8
 
 enum sa_schedule_mode {
     SA_SCHEDULE_PERSISTENT = 0, /* as many workgroups as the device holds at once, each walks many Q tiles */
@@ -150,6 +160,38 @@ int sa_mask_pack_partial(const uint8_t *mask, const int64_t mask_strides[4], int
                          int BK, const int32_t *part_ids, const int64_t part_ids_strides[4],
                          const int32_t *part_lens, const int64_t part_lens_strides[3], uint8_t *packed,
                          const int64_t packed_strides[2], void *stream);
+
+/*
+ * Classification (and optionally the packed PARTIAL tiles) of a mask that is given by a formula instead of a tensor:
+ * the same outputs as sa_mask_classify + sa_mask_pack_partial on the materialised mask, without the Sq x Sk tensor.
+ * The reference parses tensors only (mask_utils.py:85-107) and names algebraic masks, and the memory they save, as
+ * what could come next (README.md:12, :63).  With the packed tiles the forward (sa_sparse_attention_fwd_ex,
+ * mask = NULL) and the backward (q_packed / k_packed) need no mask tensor at all.
+ *
+ * Entry (b, h, q, k) attends when ANY of the n_terms terms holds; a term holds when ALL the conditions its flags
+ * switch on hold (enum sa_term_flags).  The mask does not depend on h, and on b only through the documents.
+ *
+ *   terms            HOST pointer: int32 [n_terms][8] = {flags, offset, back, ahead, q_lo, q_hi, k_lo, k_hi};
+ *                    1 <= n_terms <= SA_MAX_MASK_TERMS.  Causal: {SA_TERM_AHEAD, 0, 0, 1, ...}; causal window of w
+ *                    keys: {SA_TERM_BACK | SA_TERM_AHEAD, 0, w, 1, ...}; with Sq != Sk, offset = Sk - Sq aligns the
+ *                    last query with the last key.  The transposed mask (keys as rows) is the same formula with
+ *                    offset negated, back and ahead swapped, the ranges swapped and doc_q, doc_k swapped.
+ *   doc_q, doc_k     device int32 [B, Sq] and [B, Sk] document numbers with strides in elements (batch stride 0: shared
+ *                    by the batch), or NULL when no term has SA_TERM_SAME_DOC
+ *   lists            as in sa_mask_classify; the head stride may always be 0, the batch stride only when the documents
+ *                    do not differ between batch elements
+ *   packed           optional (NULL: lists only): as in sa_mask_pack_partial; plane (b, 0) is written for every
+ *                    distinct b, packed_strides[1] must be 0 when H > 1, base and batch stride multiples of 4 bytes
+ *   workspace        sa_mask_terms_workspace_bytes(distinct batch planes, ...) bytes of device memory
+ * BLOCK_K: a power of two >= 16.
+ */
+size_t sa_mask_terms_workspace_bytes(int distinct_b, int Sq, int Sk, int BQ, int BK);
+int sa_mask_classify_terms(const int32_t *terms, int n_terms, const int32_t *doc_q, const int64_t doc_q_strides[2],
+                           const int32_t *doc_k, const int64_t doc_k_strides[2], int B, int H, int Sq, int Sk, int BQ,
+                           int BK, int32_t *full_ids, const int64_t full_ids_strides[4], int32_t *full_lens,
+                           const int64_t full_lens_strides[3], int32_t *part_ids, const int64_t part_ids_strides[4],
+                           int32_t *part_lens, const int64_t part_lens_strides[3], uint8_t *packed,
+                           const int64_t packed_strides[2], void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Schedule of the forward: which Q tiles a workgroup processes, in order.  No counterpart in the reference, whose

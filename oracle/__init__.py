@@ -260,3 +260,39 @@ def backward_dense_fp64(q, k, v, mask, do):
     dq = np.einsum("bhqk,bhkd->bhqd", ds, k) * scale
     dk = np.einsum("bhqk,bhqd->bhkd", ds, q) * scale
     return dq, dk, dv
+
+
+def mask_from_terms(terms, B: int, Sq: int, Sk: int, doc_q=None, doc_k=None, q_rows=None) -> np.ndarray:
+    """The bool mask [B, rows, Sk] that the terms of the C ABI describe (``sa_mask_classify_terms``).
+
+    ``terms``: int [n][8] = flags, offset, back, ahead, q_lo, q_hi, k_lo, k_hi with flags 1 BACK
+    ((q + offset) - k < back), 2 AHEAD (k - (q + offset) < ahead), 4 Q_RANGE, 8 K_RANGE, 16 SAME_DOC
+    (doc_q[b, q] == doc_k[b, k]); an entry attends when any term holds, a term holds when all its flagged
+    conditions do.  The reference has no such masks (README.md:63 names them as future work); what pins this
+    function are the tensor masks it must reproduce: ``numpy.tril`` for causal, banded triangles for windows, the
+    reference's own mask semantics (mask_utils.py:34-40) through the tile totals of known masks, and a loop over
+    single entries on small shapes.  ``q_rows``: a (start, stop) range of query rows to build (all by default), so
+    that long masks can be classified strip by strip.
+    """
+    terms = np.asarray(terms, dtype=np.int64).reshape(-1, 8)
+    q_lo_, q_hi_ = (0, Sq) if q_rows is None else q_rows
+    q = np.arange(q_lo_, q_hi_, dtype=np.int64)[None, :, None]
+    k = np.arange(Sk, dtype=np.int64)[None, None, :]
+    out = np.zeros((B, q_hi_ - q_lo_, Sk), dtype=bool)
+    for flags, offset, back, ahead, q_lo, q_hi, k_lo, k_hi in terms:
+        ok = np.ones((1, q_hi_ - q_lo_, Sk), dtype=bool)
+        d = q + offset - k
+        if flags & 1:
+            ok &= d < back
+        if flags & 2:
+            ok &= -d < ahead
+        if flags & 4:
+            ok &= (q >= q_lo) & (q < q_hi)
+        if flags & 8:
+            ok &= (k >= k_lo) & (k < k_hi)
+        if flags & 16:
+            dq = np.broadcast_to(np.asarray(doc_q), (B, Sq))[:, q_lo_:q_hi_, None]
+            dk = np.broadcast_to(np.asarray(doc_k), (B, Sk))[:, None, :]
+            ok = ok & (dq == dk)
+        out |= ok
+    return out

@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsparseattn_hip.so")
 
-SA_ABI_VERSION = 10
+SA_ABI_VERSION = 11
 SA_OK = 0
 SA_ERR_INVALID_ARGUMENT = -1
 SA_ERR_UNSUPPORTED = -2
@@ -42,6 +42,8 @@ EXPORTS = (
     "sa_merge_attention_parts",
     "sa_bwd_workspace_bytes",
     "sa_sparse_attention_bwd",
+    "sa_mask_terms_workspace_bytes",
+    "sa_mask_classify_terms",
 )
 
 _lib = None
@@ -117,6 +119,13 @@ def load() -> ctypes.CDLL:
     lib.sa_sparse_attention_bwd.restype = ctypes.c_int
     lib.sa_sparse_attention_bwd.argtypes = (
         [_vp, _i64p] * 13 + [_vp, _i64p] * 8 + [_vp, ctypes.c_size_t] + [ctypes.c_int] * 6 + [ctypes.c_float, _vp]
+    )
+    lib.sa_mask_terms_workspace_bytes.restype = ctypes.c_size_t
+    lib.sa_mask_terms_workspace_bytes.argtypes = [ctypes.c_int] * 5
+    lib.sa_mask_classify_terms.restype = ctypes.c_int
+    lib.sa_mask_classify_terms.argtypes = (
+        [ctypes.POINTER(ctypes.c_int32), ctypes.c_int] + [_vp, _i64p] * 2 + [ctypes.c_int] * 6 + [_vp, _i64p] * 4
+        + [_vp, _i64p] + [_vp, ctypes.c_size_t, _vp]
     )
     if lib.sa_abi_version() != SA_ABI_VERSION:
         raise RuntimeError(f"libsparseattn_hip ABI {lib.sa_abi_version()} != expected {SA_ABI_VERSION}")

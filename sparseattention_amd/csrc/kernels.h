@@ -59,6 +59,38 @@ hipError_t launch_schedule(const ScheduleParams &p, hipStream_t stream);
 hipError_t launch_compact(const CompactParams &p, hipStream_t stream);
 hipError_t launch_pack(const PackParams &p, hipStream_t stream);
 
+// ---- masks given by a formula ---------------------------------------------------------------------
+// Entry (b, q, k) attends when any term holds; a term is the AND of the conditions its flags switch on.
+constexpr int kMaxMaskTerms = 8;
+constexpr int kTermBack = 1;      // (q + offset) - k < back
+constexpr int kTermAhead = 2;     // k - (q + offset) < ahead
+constexpr int kTermQRange = 4;    // q_lo <= q < q_hi
+constexpr int kTermKRange = 8;    // k_lo <= k < k_hi
+constexpr int kTermSameDoc = 16;  // doc_q[b][q] == doc_k[b][k]
+// A term as the kernels evaluate it: for query row q it admits the keys of
+//   [max(q + a, k_lo), min(q + b, k_hi))   when q_lo <= q < q_hi, none otherwise,
+// and of those the keys of q's document when `doc` is set.  a, b are clamped to +-2^30 and the ranges to the
+// mask's extent on the host, so that with Sq, Sk <= 2^29 everything stays inside int32.
+struct MaskTerm {
+    int32_t a, b, k_lo, k_hi, q_lo, q_hi, doc;
+};
+struct TermsParams {
+    MaskTerm terms[kMaxMaskTerms];
+    int n_terms;
+    const int32_t *doc_q, *doc_k;  // [uB, Sq] and [uB, Sk] document numbers, or null
+    int64_t dqs[2], dks[2];        // their strides in elements
+    int uB;                        // distinct planes (the mask never depends on the head)
+    int Sq, Sk, BQ, BK, nQ, nK;
+    uint8_t *cls;                  // [uB, nQ, nK] class bytes (classification)
+    // packing: the PARTIAL lists of the distinct planes and the output in PackParams layout
+    const int32_t *part_ids, *part_lens;
+    int64_t pis[4], pls[3];
+    uint8_t *packed;
+    int64_t ob;  // bytes between packed planes along b
+};
+hipError_t launch_classify_terms(const TermsParams &p, hipStream_t stream);
+hipError_t launch_pack_terms(const TermsParams &p, hipStream_t stream);
+
 // ---- block-sparse forward ------------------------------------------------------------------------
 struct FwdParams {
     const uint16_t *q, *k, *v;

@@ -450,6 +450,136 @@ int sa_mask_pack_partial(const uint8_t *mask, const int64_t mask_strides[4], int
     return SA_OK;
 }
 
+size_t sa_mask_terms_workspace_bytes(int distinct_b, int Sq, int Sk, int BQ, int BK) {
+    if (distinct_b <= 0 || check_tiling(distinct_b, 1, Sq, Sk, BQ, BK) != SA_OK) return 0;
+    return (size_t)distinct_b * (size_t)(Sq / BQ) * (size_t)(Sk / BK);
+}
+
+int sa_mask_classify_terms(const int32_t *terms, int n_terms, const int32_t *doc_q, const int64_t doc_q_strides[2],
+                           const int32_t *doc_k, const int64_t doc_k_strides[2], int B, int H, int Sq, int Sk, int BQ,
+                           int BK, int32_t *full_ids, const int64_t full_ids_strides[4], int32_t *full_lens,
+                           const int64_t full_lens_strides[3], int32_t *part_ids, const int64_t part_ids_strides[4],
+                           int32_t *part_lens, const int64_t part_lens_strides[3], uint8_t *packed,
+                           const int64_t packed_strides[2], void *workspace, size_t workspace_bytes, void *stream) {
+    g_error[0] = 0;
+    if (!terms || !full_ids || !full_ids_strides || !full_lens || !full_lens_strides || !part_ids ||
+        !part_ids_strides || !part_lens || !part_lens_strides || (doc_q && !doc_q_strides) ||
+        (doc_k && !doc_k_strides) || (packed && !packed_strides))
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_classify_terms: null pointer argument");
+    if (n_terms < 1 || n_terms > sa::kMaxMaskTerms)
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_classify_terms: %d terms (1..%d)", n_terms, sa::kMaxMaskTerms);
+    if (const int rc = check_tiling(B, H, Sq, Sk, BQ, BK)) return rc;
+    const int lbk = log2_exact(BK);
+    if (lbk < 4) return fail(SA_ERR_UNSUPPORTED, "sa_mask_classify_terms: BLOCK_K %d (supported: powers of two >= 16)", BK);
+    if ((int64_t)BQ * BK > 0x7fffffffLL)
+        return fail(SA_ERR_UNSUPPORTED, "sa_mask_classify_terms: tiles of more than 2^31-1 entries");
+
+    sa::TermsParams tp{};
+    tp.n_terms = n_terms;
+    for (int t = 0; t < n_terms; t++) {
+        const int32_t *w = terms + 8 * t;
+        if (w[0] < 0 || w[0] > 31) return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_classify_terms: term %d has unknown flags %d", t, w[0]);
+        if ((w[0] & SA_TERM_SAME_DOC) && !(doc_q && doc_k))
+            return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_classify_terms: term %d compares documents, doc_q and doc_k are needed", t);
+        // the term as an interval of keys per query row (sa::MaskTerm), in 64 bits before clamping
+        const int64_t big = (int64_t)1 << 30;
+        auto clamp = [](int64_t x, int64_t lo, int64_t hi) { return x < lo ? lo : (x > hi ? hi : x); };
+        sa::MaskTerm &m = tp.terms[t];
+        m.a = (int32_t)((w[0] & SA_TERM_BACK) ? clamp((int64_t)w[1] - w[2] + 1, -big, big) : -big);
+        m.b = (int32_t)((w[0] & SA_TERM_AHEAD) ? clamp((int64_t)w[1] + w[3], -big, big) : big);
+        m.k_lo = (int32_t)((w[0] & SA_TERM_K_RANGE) ? clamp(w[6], 0, Sk) : 0);
+        m.k_hi = (int32_t)((w[0] & SA_TERM_K_RANGE) ? clamp(w[7], 0, Sk) : Sk);
+        m.q_lo = (int32_t)((w[0] & SA_TERM_Q_RANGE) ? clamp(w[4], 0, Sq) : 0);
+        m.q_hi = (int32_t)((w[0] & SA_TERM_Q_RANGE) ? clamp(w[5], 0, Sq) : Sq);
+        m.doc = (w[0] & SA_TERM_SAME_DOC) ? 1 : 0;
+    }
+    if (Sq > (1 << 29) || Sk > (1 << 29))
+        return fail(SA_ERR_UNSUPPORTED, "sa_mask_classify_terms: more than 2^29 queries or keys");
+    // the mask depends on the batch element only through the document numbers
+    const bool per_batch = B > 1 && ((doc_q && doc_q_strides[0] != 0) || (doc_k && doc_k_strides[0] != 0));
+    const int uB = per_batch ? B : 1;
+    const int nQ = Sq / BQ, nK = Sk / BK;
+    if (nQ > 65535 || uB > 65535)
+        return fail(SA_ERR_UNSUPPORTED, "sa_mask_classify_terms: more than 65535 Q tiles or distinct mask planes");
+    const size_t need = sa_mask_terms_workspace_bytes(uB, Sq, Sk, BQ, BK);
+    if (!workspace || workspace_bytes < need)
+        return fail(SA_ERR_WORKSPACE, "sa_mask_classify_terms: workspace of %zu bytes required, %zu given", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    const int64_t ob[4] = {full_ids_strides[0], full_lens_strides[0], part_ids_strides[0], part_lens_strides[0]};
+    const int64_t oh[4] = {full_ids_strides[1], full_lens_strides[1], part_ids_strides[1], part_lens_strides[1]};
+    int zb = 0, zh = 0;
+    for (int i = 0; i < 4; i++) {
+        zb += ob[i] == 0;
+        zh += oh[i] == 0;
+    }
+    if (B > 1 && zb != 0 && (zb != 4 || per_batch))
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_classify_terms: output batch stride 0 needs a mask shared by the batch and must be 0 on all four outputs");
+    if (H > 1 && zh != 0 && zh != 4)
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_classify_terms: output head stride 0 must be 0 on all four outputs");
+    if (packed) {
+        const int64_t plane_bytes = (int64_t)Sq * Sk / 8;
+        if (!aligned(packed, 4) || packed_strides[0] % 4)
+            return fail(SA_ERR_UNSUPPORTED, "sa_mask_classify_terms: packed needs a 4-byte aligned base and batch stride");
+        if (uB > 1 && packed_strides[0] < plane_bytes)
+            return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_classify_terms: packed planes overlap (stride %lld, %lld bytes per plane)",
+                        (long long)packed_strides[0], (long long)plane_bytes);
+        if (H > 1 && packed_strides[1] != 0)
+            return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_classify_terms: the mask is the same for every head: packed_strides[1] must be 0");
+    }
+
+    tp.doc_q = doc_q;
+    tp.doc_k = doc_k;
+    for (int i = 0; i < 2; i++) {
+        tp.dqs[i] = doc_q ? doc_q_strides[i] : 0;
+        tp.dks[i] = doc_k ? doc_k_strides[i] : 0;
+    }
+    tp.uB = uB;
+    tp.Sq = Sq;
+    tp.Sk = Sk;
+    tp.BQ = BQ;
+    tp.BK = BK;
+    tp.nQ = nQ;
+    tp.nK = nK;
+    tp.cls = static_cast<uint8_t *>(workspace);
+    hipError_t e = sa::launch_classify_terms(tp, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_mask_classify_terms: classify launch failed: %s", hipGetErrorString(e));
+
+    sa::CompactParams kp{};
+    kp.cls = tp.cls;
+    kp.uH = 1;
+    kp.bcast_b = !per_batch;
+    kp.bcast_h = true;
+    kp.oB = (B > 1 && zb == 4) ? 1 : B;
+    kp.oH = (H > 1 && zh == 4) ? 1 : H;
+    kp.nQ = nQ;
+    kp.nK = nK;
+    kp.full_ids = full_ids;
+    kp.full_lens = full_lens;
+    kp.part_ids = part_ids;
+    kp.part_lens = part_lens;
+    for (int i = 0; i < 4; i++) {
+        kp.fis[i] = full_ids_strides[i];
+        kp.pis[i] = part_ids_strides[i];
+    }
+    for (int i = 0; i < 3; i++) {
+        kp.fls[i] = full_lens_strides[i];
+        kp.pls[i] = part_lens_strides[i];
+    }
+    e = sa::launch_compact(kp, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_mask_classify_terms: compaction launch failed: %s", hipGetErrorString(e));
+    if (!packed) return SA_OK;
+
+    tp.part_ids = part_ids;
+    tp.part_lens = part_lens;
+    for (int i = 0; i < 4; i++) tp.pis[i] = part_ids_strides[i];
+    for (int i = 0; i < 3; i++) tp.pls[i] = part_lens_strides[i];
+    tp.packed = packed;
+    tp.ob = packed_strides[0];
+    e = sa::launch_pack_terms(tp, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_mask_classify_terms: packing launch failed: %s", hipGetErrorString(e));
+    return SA_OK;
+}
+
 int sa_decode_num_splits(int B, int H, int Sq, int Sk, int BK) {
     if (B <= 0 || H <= 0 || Sq <= 0 || Sq > 32 || Sk <= 0 || BK < 32 || Sk % BK) return 0;
     int dev = 0, cus = 0;

@@ -5,8 +5,9 @@ Mirrors the interface of the reference's ``sparseattention/mask_utils.py``:
 """
 from __future__ import annotations
 
+import ctypes
 from dataclasses import dataclass
-from typing import Optional
+from typing import Optional, Sequence, Tuple
 
 import torch
 
@@ -83,6 +84,32 @@ def compute_mask_slow(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int) -> MaskMet
     return MaskMetadata(fid, fl, pid, pl)
 
 
+def _make_schedule(lib, fl, pl, B, H, Sq, Sk, BLOCK_Q, BLOCK_K, schedule, dev):
+    """(schedule tensor, mode) for ``compute_mask_kernel(..., schedule=...)``; (None, 0) without one."""
+    if not schedule:
+        return None, 0
+    modes = {"persistent": _native.SA_SCHEDULE_PERSISTENT, "pairs": _native.SA_SCHEDULE_PAIRS,
+             True: _native.SA_SCHEDULE_PAIRS}
+    if schedule not in modes:
+        raise ValueError(f"schedule must be 'pairs', 'persistent' or None (got {schedule!r})")
+    mode = modes[schedule]
+    nQ = Sq // BLOCK_Q
+    nbytes = int(lib.sa_fwd_schedule_bytes(B, H, Sq, Sk, BLOCK_Q, BLOCK_K, mode))
+    if nbytes == 0:
+        raise ValueError(f"no scheduled forward for BLOCK_Q={BLOCK_Q}, BLOCK_K={BLOCK_K}, Sk={Sk}")
+    sched = torch.empty(nbytes // 4, dtype=torch.int32, device=dev)
+    rc = lib.sa_fwd_schedule(fl.data_ptr(), _native.strides(fl.stride()), pl.data_ptr(),
+                             _native.strides(pl.stride()), B, H, Sq, Sk, BLOCK_Q, BLOCK_K, mode,
+                             sched.data_ptr(), nbytes, torch.cuda.current_stream(dev).cuda_stream)
+    _native.check(rc)
+    if mode == _native.SA_SCHEDULE_PAIRS:
+        sched = sched.view(-1, 3, 4)
+    else:
+        G = min(2 * torch.cuda.get_device_properties(dev).multi_processor_count, 512) & ~7
+        sched = sched.view(G, nbytes // (16 * G), 4)
+    return sched, mode
+
+
 def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int, pack_partial: Optional[bool] = None,
                         schedule=None) -> MaskMetadata:
     """Classify the mask's tiles on the GPU (replaces mask_utils.py:85-107).
@@ -145,27 +172,7 @@ def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int, pack_par
             )
             _native.check(rc)
             packed = packed.expand(B, H, nQ, nK, BLOCK_Q * BLOCK_K // 8)
-        sched = None
-        mode = 0
-        if schedule:
-            modes = {"persistent": _native.SA_SCHEDULE_PERSISTENT, "pairs": _native.SA_SCHEDULE_PAIRS,
-                     True: _native.SA_SCHEDULE_PAIRS}
-            if schedule not in modes:
-                raise ValueError(f"schedule must be 'pairs', 'persistent' or None (got {schedule!r})")
-            mode = modes[schedule]
-            nbytes = int(lib.sa_fwd_schedule_bytes(B, H, Sq, Sk, BLOCK_Q, BLOCK_K, mode))
-            if nbytes == 0:
-                raise ValueError(f"no scheduled forward for BLOCK_Q={BLOCK_Q}, BLOCK_K={BLOCK_K}, Sk={Sk}")
-            sched = torch.empty(nbytes // 4, dtype=torch.int32, device=dev)
-            rc = lib.sa_fwd_schedule(fl.data_ptr(), _native.strides(fl.stride()), pl.data_ptr(),
-                                     _native.strides(pl.stride()), B, H, Sq, Sk, BLOCK_Q, BLOCK_K, mode,
-                                     sched.data_ptr(), nbytes, torch.cuda.current_stream(dev).cuda_stream)
-            _native.check(rc)
-            if mode == _native.SA_SCHEDULE_PAIRS:
-                sched = sched.view(-1, 3, 4)
-            else:
-                G = min(2 * torch.cuda.get_device_properties(dev).multi_processor_count, 512) & ~7
-                sched = sched.view(G, nbytes // (16 * G), 4)
+        sched, mode = _make_schedule(lib, fl, pl, B, H, Sq, Sk, BLOCK_Q, BLOCK_K, schedule, dev)
     return MaskMetadata(fid, fl, pid, pl, packed, sched, mode)
 
 
@@ -209,3 +216,144 @@ def select_block_sizes(mask: torch.Tensor, candidates=DEFAULT_TILE_CANDIDATES, p
     if best is None:
         raise ValueError(f"no candidate tile size divides a mask of shape {tuple(mask.shape)}")
     return best[1], best[2], best[3], report
+
+
+# ---- masks given by a formula -----------------------------------------------------------------------------------
+_TERM_BACK, _TERM_AHEAD, _TERM_Q_RANGE, _TERM_K_RANGE, _TERM_SAME_DOC = 1, 2, 4, 8, 16
+MAX_MASK_TERMS = 8
+
+
+@dataclass(frozen=True)
+class MaskTerm:
+    """One term of a mask given by a formula: the AND of the conditions that are set.
+
+    ``back``: ``(q + offset) - k < back`` (how far behind the diagonal a key may lie); ``ahead``:
+    ``k - (q + offset) < ahead`` (1: causal); ``q_range`` / ``k_range``: half-open index ranges; ``same_doc``:
+    ``doc_q[b, q] == doc_k[b, k]``.  A mask is the OR of up to ``MAX_MASK_TERMS`` terms.  The reference takes tensor
+    masks only and lists "algebraically defined masks ... to avoid materialisation + memory costs" as what could come
+    next (README.md:63).
+    """
+
+    back: Optional[int] = None
+    ahead: Optional[int] = None
+    offset: int = 0
+    q_range: Optional[Tuple[int, int]] = None
+    k_range: Optional[Tuple[int, int]] = None
+    same_doc: bool = False
+
+    def encode(self):
+        """The eight int32 of the C ABI: flags, offset, back, ahead, q_lo, q_hi, k_lo, k_hi."""
+        flags = ((_TERM_BACK if self.back is not None else 0) | (_TERM_AHEAD if self.ahead is not None else 0)
+                 | (_TERM_Q_RANGE if self.q_range is not None else 0) | (_TERM_K_RANGE if self.k_range is not None else 0)
+                 | (_TERM_SAME_DOC if self.same_doc else 0))
+        q_lo, q_hi = self.q_range if self.q_range is not None else (0, 0)
+        k_lo, k_hi = self.k_range if self.k_range is not None else (0, 0)
+        return [flags, int(self.offset), int(self.back or 0), int(self.ahead or 0), int(q_lo), int(q_hi), int(k_lo), int(k_hi)]
+
+    def transposed(self) -> "MaskTerm":
+        """The same condition with keys as rows: term(q, k) == term.transposed()(k, q)."""
+        return MaskTerm(back=self.ahead, ahead=self.back, offset=-self.offset, q_range=self.k_range,
+                        k_range=self.q_range, same_doc=self.same_doc)
+
+
+def causal_term(window: Optional[int] = None, offset: int = 0, same_doc: bool = False) -> MaskTerm:
+    """``k <= q + offset``, optionally only the last ``window`` such keys, optionally within one document."""
+    return MaskTerm(back=window, ahead=1, offset=offset, same_doc=same_doc)
+
+
+def block_term(q_range: Optional[Tuple[int, int]] = None, k_range: Optional[Tuple[int, int]] = None) -> MaskTerm:
+    """Every (q, k) with q and k in the given half-open ranges (None: all), e.g. a bidirectional prefix or sink keys."""
+    return MaskTerm(q_range=q_range, k_range=k_range)
+
+
+def _check_docs(doc, B, S, name):
+    if doc is None:
+        return None
+    if doc.dim() == 1:
+        doc = doc[None]
+    if doc.dim() != 2 or doc.shape[-1] != S or doc.shape[0] not in (1, B) or doc.dtype != torch.int32:
+        raise ValueError(f"{name}: expected int32 [{B},{S}] or [{S}], got {doc.dtype} {tuple(doc.shape)}")
+    return doc.expand(B, S)
+
+
+def materialize_mask_terms(terms: Sequence[MaskTerm], B: int, Sq: int, Sk: int, doc_q=None, doc_k=None, device=None):
+    """The bool mask [B,1,Sq,Sk] (or [1,1,Sq,Sk] without documents) that the terms describe, in plain torch: for
+    checks, for the decode path (which reads a tensor) and for :func:`torch.nn.functional.scaled_dot_product_attention`."""
+    doc_q, doc_k = _check_docs(doc_q, B, Sq, "doc_q"), _check_docs(doc_k, B, Sk, "doc_k")
+    if device is None:
+        device = doc_q.device if doc_q is not None else "cpu"
+    q = torch.arange(Sq, device=device, dtype=torch.int64)[:, None]
+    k = torch.arange(Sk, device=device, dtype=torch.int64)[None, :]
+    out = torch.zeros(B if doc_q is not None else 1, 1, Sq, Sk, dtype=torch.bool, device=device)
+    for t in terms:
+        ok = torch.ones(1, 1, Sq, Sk, dtype=torch.bool, device=device)
+        d = q + t.offset - k
+        if t.back is not None:
+            ok = ok & (d < t.back)
+        if t.ahead is not None:
+            ok = ok & (-d < t.ahead)
+        if t.q_range is not None:
+            ok = ok & (q >= t.q_range[0]) & (q < t.q_range[1])
+        if t.k_range is not None:
+            ok = ok & (k >= t.k_range[0]) & (k < t.k_range[1])
+        if t.same_doc:
+            if doc_q is None or doc_k is None:
+                raise ValueError("a term with same_doc needs doc_q and doc_k")
+            ok = ok & (doc_q[:, None, :, None] == doc_k[:, None, None, :])
+        out = out | ok
+    return out
+
+
+def compute_mask_terms(terms: Sequence[MaskTerm], B: int, H: int, Sq: int, Sk: int, BLOCK_Q: int, BLOCK_K: int,
+                       doc_q: Optional[torch.Tensor] = None, doc_k: Optional[torch.Tensor] = None, device=None,
+                       pack_partial: bool = True, schedule=None) -> MaskMetadata:
+    """:func:`compute_mask_kernel` for a mask given by terms: the same lists (and packed PARTIAL tiles, schedule) as
+    for ``materialize_mask_terms(...)``, computed on the GPU from the formula without the Sq x Sk tensor.
+
+    With ``pack_partial`` the result carries everything the forward needs: ``sparse_attention(q, k, v, None, BLOCK_Q,
+    BLOCK_K, mask_metadata=md)``.  ``doc_q`` / ``doc_k``: int32 document numbers [B,Sq] / [B,Sk] (or [Sq] / [Sk]) on
+    the GPU for terms with ``same_doc``.  ``device``: where to compute when there are no documents.
+    """
+    terms = list(terms)
+    if not 1 <= len(terms) <= MAX_MASK_TERMS:
+        raise ValueError(f"1..{MAX_MASK_TERMS} terms (got {len(terms)})")
+    assert Sq % BLOCK_Q == 0, "Sq must be a multiple of BLOCK_Q"
+    assert Sk % BLOCK_K == 0, "Sk must be a multiple of BLOCK_K"
+    doc_q, doc_k = _check_docs(doc_q, B, Sq, "doc_q"), _check_docs(doc_k, B, Sk, "doc_k")
+    if any(t.same_doc for t in terms) and (doc_q is None or doc_k is None):
+        raise ValueError("a term with same_doc needs doc_q and doc_k")
+    dev = torch.device(device) if device is not None else (doc_q.device if doc_q is not None else torch.device("cuda"))
+    if dev.type != "cuda" or any(d is not None and d.device != dev for d in (doc_q, doc_k)):
+        raise RuntimeError("compute_mask_terms runs on a ROCm GPU (documents on the same device); "
+                           "materialize_mask_terms + compute_mask_slow run anywhere")
+    lib = _native.load()
+    nQ, nK = Sq // BLOCK_Q, Sk // BLOCK_K
+    per_batch = B > 1 and any(d is not None and d.stride(0) != 0 for d in (doc_q, doc_k))
+    uB = B if per_batch else 1
+    flat = [w for t in terms for w in t.encode()]
+    c_terms = (ctypes.c_int32 * len(flat))(*flat)
+    S = _native.strides
+    with torch.cuda.device(dev):
+        fid = torch.empty(uB, 1, nQ, nK, dtype=torch.int32, device=dev).expand(B, H, nQ, nK)
+        pid = torch.empty(uB, 1, nQ, nK, dtype=torch.int32, device=dev).expand(B, H, nQ, nK)
+        fl = torch.empty(uB, 1, nQ, dtype=torch.int32, device=dev).expand(B, H, nQ)
+        pl = torch.empty(uB, 1, nQ, dtype=torch.int32, device=dev).expand(B, H, nQ)
+        packed = None
+        if pack_partial:
+            packed = torch.empty(uB, 1, nQ, nK, BLOCK_Q * BLOCK_K // 8, dtype=torch.uint8, device=dev)
+            packed = packed.expand(B, H, nQ, nK, BLOCK_Q * BLOCK_K // 8)
+        need = int(lib.sa_mask_terms_workspace_bytes(uB, Sq, Sk, BLOCK_Q, BLOCK_K))
+        workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+        rc = lib.sa_mask_classify_terms(
+            c_terms, len(terms),
+            doc_q.data_ptr() if doc_q is not None else None, S(doc_q.stride()) if doc_q is not None else None,
+            doc_k.data_ptr() if doc_k is not None else None, S(doc_k.stride()) if doc_k is not None else None,
+            B, H, Sq, Sk, BLOCK_Q, BLOCK_K,
+            fid.data_ptr(), S(fid.stride()), fl.data_ptr(), S(fl.stride()),
+            pid.data_ptr(), S(pid.stride()), pl.data_ptr(), S(pl.stride()),
+            packed.data_ptr() if packed is not None else None, S(packed.stride()[:2]) if packed is not None else None,
+            workspace.data_ptr(), workspace.numel(), torch.cuda.current_stream(dev).cuda_stream)
+        _native.check(rc)
+        del workspace
+        sched, mode = _make_schedule(lib, fl, pl, B, H, Sq, Sk, BLOCK_Q, BLOCK_K, schedule, dev)
+    return MaskMetadata(fid, fl, pid, pl, packed, sched, mode)

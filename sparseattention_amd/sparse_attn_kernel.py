@@ -6,7 +6,7 @@ import math
 import torch
 
 from . import _native
-from .mask_utils import MaskMetadata, compute_mask_kernel
+from .mask_utils import MaskMetadata, compute_mask_kernel, compute_mask_terms
 
 _DTYPES = {torch.bfloat16: _native.SA_DTYPE_BF16, torch.float16: _native.SA_DTYPE_FP16}
 
@@ -17,7 +17,7 @@ def _kernel_ready(t: torch.Tensor) -> torch.Tensor:
     return t if ok else t.contiguous()
 
 
-def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor, BLOCK_Q, BLOCK_K,
+def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor | None, BLOCK_Q, BLOCK_K,
                      mask_metadata: MaskMetadata | None = None, *, return_lse: bool = False):
     """softmax(q kᵀ / sqrt(D) + (mask ? 0 : -inf)) v, skipping KV tiles the mask empties.
 
@@ -28,6 +28,8 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
     Returns ``o`` with q's shape, dtype and strides; with ``return_lse=True`` (not in the reference, which drops
     the row statistics after the division at sparse_attn_kernel.py:144) the pair ``(o, lse)`` where ``lse``
     [B,H,Sq] float32 is the log of the row's softmax denominator, -inf for rows that attend to nothing.
+    ``mask`` may be None when ``mask_metadata`` carries ``packed_masks`` (the kernels then read no mask tensor), which
+    is how masks given by a formula run (:func:`compute_mask_terms`).
     """
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be [B,H,S,D]")
@@ -39,13 +41,16 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
         raise RuntimeError("sparse_attention needs q, k, v on a ROCm GPU; there is no CPU path")
     if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
         raise TypeError(f"q, k, v must share dtype bfloat16 or float16 (got {q.dtype}, {k.dtype}, {v.dtype})")
+    if mask is None and getattr(mask_metadata, "packed_masks", None) is None:
+        raise ValueError("sparse_attention without a mask tensor needs mask_metadata with packed_masks")
     if (Sq == BLOCK_Q and Sq < 32 and BLOCK_K >= 32 and getattr(mask_metadata, "packed_masks", None) is None
             and getattr(mask_metadata, "schedule", None) is None):
         # one Q tile of fewer rows than the forward kernels tile by: the split-KV kernels
         return sparse_attention_decode(q, k, v, mask, BLOCK_K, mask_metadata, return_lse=return_lse)
     sm_scale = D ** (-0.5) * 1 / math.log(2)  # exp2 replaces exp (sparse_attn_kernel.py:152)
 
-    mask = mask.expand(B, H, Sq, Sk)
+    if mask is not None:
+        mask = mask.expand(B, H, Sq, Sk)
 
     if mask_metadata is None:
         mask_metadata = compute_mask_kernel(mask, BLOCK_Q, BLOCK_K)
@@ -56,9 +61,10 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
                            ("unmasked_lens", fl, (B, H, nQ)), ("masked_lens", pl, (B, H, nQ))):
         if tuple(t.shape) != shape or t.dtype != torch.int32 or t.device != q.device:
             raise ValueError(f"mask_metadata.{name}: expected int32 {shape} on {q.device}, got {t.dtype} {tuple(t.shape)} on {t.device}")
-    assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
-    if mask.device != q.device:
-        raise ValueError("mask must be on the same device as q")
+    if mask is not None:
+        assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
+        if mask.device != q.device:
+            raise ValueError("mask must be on the same device as q")
     packed = getattr(mask_metadata, "packed_masks", None)
     if packed is not None:
         shape = (B, H, nQ, nK, BLOCK_Q * BLOCK_K // 8)
@@ -77,7 +83,8 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
     S = _native.strides
     with torch.cuda.device(q.device):
         common = (qc.data_ptr(), S(qc.stride()), kc.data_ptr(), S(kc.stride()), vc.data_ptr(), S(vc.stride()),
-                  o.data_ptr(), S(o.stride()), mask.data_ptr(), S(mask.stride()),
+                  o.data_ptr(), S(o.stride()),
+                  mask.data_ptr() if mask is not None else None, S(mask.stride()) if mask is not None else None,
                   fid.data_ptr(), S(fid.stride()), fl.data_ptr(), S(fl.stride()),
                   pid.data_ptr(), S(pid.stride()), pl.data_ptr(), S(pl.stride()))
         tail = (B, H, Sq, Sk, D, int(BLOCK_Q), int(BLOCK_K), _DTYPES[q.dtype], sm_scale,
@@ -184,6 +191,17 @@ def compute_backward_metadata(mask: torch.Tensor, pack_partial: bool = True) -> 
     return BackwardMetadata(compute_mask_kernel(mask, 128, 64, pack_partial=pack_partial),
                             compute_mask_kernel(transposed, 128, 64, pack_partial=pack_partial),
                             None if pack_partial else transposed)
+
+
+def compute_backward_metadata_terms(terms, B: int, H: int, Sq: int, Sk: int, doc_q=None, doc_k=None,
+                                    device=None) -> BackwardMetadata:
+    """:func:`compute_backward_metadata` for a mask given by terms (:func:`compute_mask_terms`): both tilings with
+    their packed PARTIAL tiles, the key-major one from the transposed terms, so that
+    ``sparse_attention_backward(..., mask=None, bwd_metadata=...)`` runs without any mask tensor."""
+    terms = list(terms)
+    return BackwardMetadata(
+        compute_mask_terms(terms, B, H, Sq, Sk, 128, 64, doc_q, doc_k, device),
+        compute_mask_terms([t.transposed() for t in terms], B, H, Sk, Sq, 128, 64, doc_k, doc_q, device), None)
 
 
 def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor,
