@@ -43,6 +43,9 @@ TRAFFIC_FWD_CAUSAL_BYTES = 1.3566e9      # 1037.8 MiB read + 256.0 MiB written
 TRAFFIC_CLASSIFY_1GIB_BYTES = 1.0744e9   # 1,048,622 + 327 KiB read, 256 + 45.5 KiB written
 # decode workloads (profiles/sparse_decode_kernel_B8H32Sk32768D128.txt), both kernels
 TRAFFIC_DECODE_BYTES = (4.2959e9, 1.6225e9)
+# backward of the headline workload (profiles/sparse_bwd_kernel_causal_B8H32S4096D128.txt), three passes + prepare:
+# 4256 MiB read + 778.7 MiB written
+TRAFFIC_BWD_CAUSAL_BYTES = 5.280e9
 
 B, H, S, D = 8, 32, 4096, 128
 BQ, BK = 128, 32
@@ -222,7 +225,7 @@ def backward_case(q, k, v, steps, warmup):
         "ms": round(wall_ms, 4), "kernel_ms": round(ev_ms, 4),
         "executed_tflops": round(executed / (ev_ms * 1e-3) / 1e12, 1),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BWD_CAUSAL_BYTES,
                      "kernel": "sparse_bwd_kernel x3 (+ bwd_prepare_kernel)", "flop_per_launch": algorithmic},
     }
 
