@@ -121,7 +121,8 @@ int sa_mask_classify(const uint8_t *mask, const int64_t mask_strides[4], int B, 
  * mask applied, online softmax state in fp32, P rounded to the input dtype before P.V
  * (sparse_attn_kernel.py:61).  Rows with no attended key produce 0 (the reference produces NaN).
  *
- * Supported: D in {64,128}; BQ in {32,64,128,256}; BK a power of two >= 16.
+ * Supported: D in {64,128,256}; BQ in {32,64,128,256} (64 and 128 at D = 256, where a given schedule is not used);
+ * BK a power of two >= 16.
  * ids[..., :len] must hold valid KV-tile indices (< Sk/BK): they address K and V directly.
  */
 int sa_sparse_attention_fwd(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],

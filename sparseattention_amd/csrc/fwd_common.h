@@ -118,11 +118,11 @@ __device__ __forceinline__ void dma16(const void *base, uint32_t lane_offset, ui
 //   V: the 4 rows touched by one half-wave transposing read fall into 4 different 64-byte bank groups.
 template <int D>
 __device__ __forceinline__ int k_swizzle(int row) {
-    return D == 128 ? (row & 15) : ((row >> 1) & 7);
+    return D >= 128 ? (row & 15) : ((row >> 1) & 7);
 }
 template <int D>
 __device__ __forceinline__ int v_swizzle(int row) {
-    return D == 128 ? 4 * (row & 3) : 4 * ((row >> 1) & 1);
+    return D >= 128 ? 4 * (row & 3) : 4 * ((row >> 1) & 1);
 }
 
 // log2-domain slack before the running maximum is raised (and the accumulator rescaled).  Scores are

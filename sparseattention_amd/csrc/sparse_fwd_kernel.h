@@ -59,7 +59,7 @@ __device__ __forceinline__ void wait_vm_at_most(int n, int step) {
 // lists of the tiles after that are on their way, so that the latencies a fresh workgroup would pay one after
 // the other (arguments, counts, lists, first K/V chunk) are paid once per workgroup instead of once per tile.
 template <int DT, int D, int NW, int MODE, int NS, bool PP, bool PK, bool PS>
-__global__ __launch_bounds__(NW * 64, NW >= 4 ? 2 : 1) void sparse_fwd_kernel(const FwdParams p) {
+__global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse_fwd_kernel(const FwdParams p) {
     static_assert(!PS || (!PP && NS == 2), "persistent workgroups use the two-stage loop");
     using E = Elem<DT>;
     constexpr int ROWB = D * 2;                   // bytes per K/V row in LDS
@@ -985,11 +985,14 @@ hipError_t launch_mode(const FwdParams &p, hipStream_t stream) {
 template <int DT, int D, bool PK, bool PS>
 hipError_t launch_bq(const FwdParams &p, int BQ, hipStream_t stream) {
     switch (BQ) {
-        case 32: return launch_mode<DT, D, 1, PK, PS>(p, stream);
+        case 32:
+            if constexpr (D > 128) return hipErrorInvalidValue;  // a lone wave would spill its registers there
+            else return launch_mode<DT, D, 1, PK, PS>(p, stream);
         case 64: return launch_mode<DT, D, 2, PK, PS>(p, stream);
         case 128: return launch_mode<DT, D, 4, PK, PS>(p, stream);
         case 256:
-            if constexpr (PS) return hipErrorInvalidValue;  // 8-wave workgroups are not persistent
+            // 8-wave workgroups are not persistent, and their four stages do not fit the LDS at D = 256
+            if constexpr (PS || D > 128) return hipErrorInvalidValue;
             else return launch_mode<DT, D, 8, PK, false>(p, stream);
         default: return hipErrorInvalidValue;
     }
@@ -1005,6 +1008,11 @@ hipError_t launch_fwd_variant(const FwdParams &p, int D, int BQ, hipStream_t str
     switch (D) {
         case 64: return launch_bq<DT, 64, PK, PS>(p, BQ, stream);
         case 128: return launch_bq<DT, 128, PK, PS>(p, BQ, stream);
+        case 256:
+            // one workgroup per CU (its two stages of K and V take 128 KiB of LDS) with the whole register file:
+            // one wave per SIMD; no schedules
+            if constexpr (PS) return hipErrorInvalidValue;
+            else return launch_bq<DT, 256, PK, false>(p, BQ, stream);
         default: return hipErrorInvalidValue;
     }
 }

@@ -196,9 +196,12 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
         return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd: sm_scale_log2 must be positive and finite");
     if (dtype != SA_DTYPE_BF16 && dtype != SA_DTYPE_FP16)
         return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: dtype code %d (supported: 0 = bf16, 1 = fp16)", dtype);
-    if (D != 64 && D != 128) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: head dim %d (supported: 64, 128)", D);
+    if (D != 64 && D != 128 && D != 256)
+        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: head dim %d (supported: 64, 128, 256)", D);
     if (BQ != 32 && BQ != 64 && BQ != 128 && BQ != 256)
         return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: BLOCK_Q %d (supported: 32, 64, 128, 256)", BQ);
+    if (D == 256 && BQ != 64 && BQ != 128)
+        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: BLOCK_Q %d at head dim 256 (supported there: 64, 128)", BQ);
     const int lbk = log2_exact(BK);
     if (lbk < 4) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: BLOCK_K %d (supported: powers of two >= 16)", BK);
     const int64_t *st[4] = {q_strides, k_strides, v_strides, o_strides};
@@ -243,7 +246,7 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
     fp.pks[1] = use_packed ? packed_strides[1] : 0;
     fp.nK = Sk / BK;
     fp.sched = nullptr;
-    if (schedule) {
+    if (schedule && D <= 128) {  // head dim 256 has no scheduled kernels; the order of Q tiles does not change results
         int G = 0, R = 0;
         const size_t want = schedule_shape(B, H, Sq, Sk, BQ, BK, schedule_mode, &G, &R);
         if (want != 0 && want == schedule_bytes) {

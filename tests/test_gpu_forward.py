@@ -309,3 +309,45 @@ def test_lse_output(gpu, route, BQ, BK):
     # the row sum adds up P as rounded to bf16 (8 significant bits) for the P.V product: a sum that one term
     # dominates is off by up to 2^-8 of itself
     assert (lse[live].double() - want[live]).abs().max() <= 6e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("BQ", [64, 128])
+@pytest.mark.parametrize("BK", [16, 32, 64, 256])
+def test_head_dim_256(gpu, BQ, BK, dtype):
+    # one workgroup per CU with the whole register file; bool-mask reads, packed tiles, lse, a schedule that is ignored
+    B, H, Sq, Sk, D = 2, 2, 384, 768, 256
+    q, _, _ = W.qkv(B, H, Sq, D, dtype, seed=BQ + BK, device=gpu)
+    _, k, v = W.qkv(B, H, Sk, D, dtype, seed=BQ * BK, device=gpu)
+    coarse = torch.rand(B, 1, Sq // 32, Sk // 32, generator=torch.Generator().manual_seed(BK)) < 0.5
+    fine = torch.rand(B, 1, Sq, Sk, generator=torch.Generator().manual_seed(BQ)) < 0.7
+    mask = (coarse.repeat_interleave(32, 2).repeat_interleave(32, 3) & fine).to(gpu)
+    mask[..., :16] = True
+    me = mask.expand(B, H, Sq, Sk)
+    o = sparse_attention(q, k, v, me, BQ, BK, compute_mask_kernel(me, BQ, BK, pack_partial=False))
+    want = oracle_out(q, k, v, mask, BQ, BK, p_round=1 if dtype == torch.bfloat16 else 2)
+    err = (o.float().cpu() - want).abs()
+    assert err.max() <= TOL and err.mean() <= 1e-3, f"vs oracle: max {err.max()}, mean {err.mean()}"
+    ref = sdpa32(q, k, v, mask)
+    assert (o.float() - ref).abs().max() <= TOL
+    sched = "pairs" if BK <= 64 else None
+    o2, lse = sparse_attention(q, k, v, None, BQ, BK, compute_mask_kernel(me, BQ, BK, pack_partial=True, schedule=sched),
+                               return_lse=True)
+    assert torch.equal(o, o2)
+    s = torch.einsum("bhqd,bhkd->bhqk", q.float(), k.float()) / math.sqrt(D)
+    want_lse = torch.logsumexp(s.masked_fill(~me, float("-inf")), dim=-1)
+    assert (lse - want_lse).abs().max() <= 6e-3
+
+
+def test_head_dim_256_limits_and_long_rows(gpu):
+    qb = torch.zeros(1, 1, 256, 256, dtype=torch.bfloat16, device=gpu)
+    m = torch.ones(256, 256, dtype=torch.bool, device=gpu)
+    for BQ in (32, 256):
+        with pytest.raises(_native.SparseAttnError, match="head dim 256"):
+            sparse_attention(qb, qb, qb, m, BQ, 32)
+    # causal, 4096 keys: long lists, every plane against fp32 SDPA
+    B, H, S, D = 1, 4, 4096, 256
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=77, device=gpu)
+    mask = W.causal_mask(S, gpu)
+    o = sparse_attention(q, k, v, mask, 128, 32)
+    assert (o.float() - sdpa32(q, k, v, mask)).abs().max() <= TOL
