@@ -5,7 +5,7 @@
 
 A step is one forward pass (sa_sparse_attention_fwd_ex) over the headline workload: causal bool mask
 passed as a tensor, B=8 H=32 S=4096 D=128 bf16, tiles 128x32, inputs and the precomputed mask metadata
-(tile lists, bit-packed partial tiles, pairs schedule: what compute_mask_kernel returns) resident in HBM;
+(tile lists and bit-packed partial tiles: what compute_mask_kernel returns by default) resident in HBM;
 the reference also excludes preprocessing from the forward time and reports it separately
 (test_attn.py:38,65,68).  Prints ONE JSON line.
 
@@ -15,7 +15,7 @@ the reference also excludes preprocessing from the forward time and reports it s
              (full + partial tiles) * 4*BQ*BK*D flop per launch / mean launch duration (HIP events)
   mask_classify   the preprocessing kernels on a 1 GiB mask against the HBM peak
   across_p   the same forward on random block masks of sparsity p, a dense mask and the causal one
-  variants   the headline workload through the other routes of the library (bool-mask reads, no schedule,
+  variants   the headline workload through the other routes of the library (bool-mask reads, the pairs schedule,
              persistent workgroups)
   backward   dq, dk, dv of the headline workload (sparse_attention_backward) against the MFMA peak
   decode     the split-KV kernels for few query rows (sparse_attention_decode) against the HBM peak: K and V of
@@ -39,7 +39,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E peak, GB/s
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this script and scaled by
 # the readings of a 1 GiB device copy in the same run (--calibrate-copy).  The summaries with the commands
 # are profiles/sparse_fwd_kernel_causal_B8H32S4096D128.txt and profiles/mask_classify_kernels_mask_32768x32768.txt.
-TRAFFIC_FWD_CAUSAL_BYTES = 1.3566e9      # 1037.8 MiB read + 256.0 MiB written
+TRAFFIC_FWD_CAUSAL_BYTES = 1.2644e9      # 949.1 MiB read + 256.8 MiB written
 TRAFFIC_CLASSIFY_1GIB_BYTES = 1.0744e9   # 1,048,622 + 327 KiB read, 256 + 45.5 KiB written
 # decode workloads (profiles/sparse_decode_kernel_B8H32Sk32768D128.txt), both kernels
 TRAFFIC_DECODE_BYTES = (4.2959e9, 1.6225e9)
@@ -335,7 +335,7 @@ def main():
     torch.cuda.set_device(0)
     q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=0, device="cuda")
 
-    head = forward_case("causal", W.causal_mask(S, "cuda"), q, k, v, args.steps, args.warmup, schedule="pairs")
+    head = forward_case("causal", W.causal_mask(S, "cuda"), q, k, v, args.steps, args.warmup)
     achieved = head["_executed_flop"] / (head["kernel_ms"] * 1e-3) / 1e12
     result = {
         "metric": "effective TFLOP/s of the block-sparse forward (4*B*H*S*S*D*mean(mask)/time), B8 H32 S4096 D128 bf16",
@@ -352,7 +352,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "configs[1]: causal bool mask [4096,4096] passed as a tensor, B=8 H=32 S=4096 D=128 bf16, "
                                "q/k/v ~ N(0,1), tiles BLOCK_Q=128 BLOCK_K=32, mask metadata precomputed "
-                               "(tile lists, bit-packed partial tiles, pairs schedule)",
+                               "(tile lists, bit-packed partial tiles; one workgroup per Q tile)",
                    "executed_tiles_per_plane": int(head["_executed_flop"] // (B * H * FLOP_PER_TILE)),
                    "partial_tiles_per_plane": head["partial_tiles_per_plane"]},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
