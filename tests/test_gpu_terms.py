@@ -143,3 +143,40 @@ def test_argument_errors(gpu):
     assert lib.sa_mask_terms_workspace_bytes(0, 256, 512, 128, 32) == 0
     with pytest.raises(_native.SparseAttnError):  # BLOCK_K below 16
         compute_mask_terms([causal_term()], 1, 1, 128, 128, 128, 8, device=gpu)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_seeded_random_terms(gpu, seed):
+    # random flags and values (negative and huge offsets, ranges past the extents, empty ranges, unsorted documents),
+    # random tilings and lengths: the decisions taken from the first and last row of a tile must agree with the
+    # entry-by-entry tensor path everywhere
+    g = torch.Generator().manual_seed(1000 + seed)
+    ri = lambda lo, hi: int(torch.randint(lo, hi, (1,), generator=g))
+    BQ, BK = [(128, 32), (64, 16), (32, 64), (16, 128), (256, 32), (128, 256)][seed % 6]
+    B, H = ri(1, 4), ri(1, 3)
+    Sq, Sk = BQ * ri(1, 5), max(BK, 64) * ri(1, 6)
+    n_docs = ri(1, 6)
+    if seed % 3 == 0:  # contiguous documents of random lengths
+        dk = torch.sort(torch.randint(0, n_docs, (B, Sk), generator=g), dim=1).values.int()
+        dq = torch.sort(torch.randint(0, n_docs, (B, Sq), generator=g), dim=1).values.int()
+    elif seed % 3 == 1:  # blocks of 32 positions with arbitrary document numbers
+        dk = torch.randint(0, n_docs, (B, (Sk + 31) // 32), generator=g).repeat_interleave(32, 1)[:, :Sk].int()
+        dq = torch.randint(0, n_docs, (B, (Sq + 31) // 32), generator=g).repeat_interleave(32, 1)[:, :Sq].int()
+    else:  # one layout for the whole batch
+        dk = torch.sort(torch.randint(0, n_docs, (1, Sk), generator=g), dim=1).values.int()
+        dq = torch.sort(torch.randint(0, n_docs, (1, Sq), generator=g), dim=1).values.int()
+    dq, dk = dq.to(gpu), dk.to(gpu)
+    big = [2 ** 31 - 1, -2 ** 31, 2 ** 30, -2 ** 30 - 5]
+    val = lambda span: big[ri(0, 4)] if ri(0, 12) == 0 else ri(-span, span + 1)
+    terms = []
+    for _ in range(ri(1, 5)):
+        rng = lambda S: tuple(sorted((ri(-20, S + 20), ri(-20, S + 20)))) if ri(0, 3) else (ri(0, S), ri(0, S))
+        terms.append(MaskTerm(back=val(Sk) if ri(0, 2) else None, ahead=val(Sk // 2) if ri(0, 2) else None,
+                              offset=val(Sk) if ri(0, 2) else 0, q_range=rng(Sq) if ri(0, 3) == 0 else None,
+                              k_range=rng(Sk) if ri(0, 3) == 0 else None, same_doc=ri(0, 3) == 0))
+    md = compute_mask_terms(terms, B, H, Sq, Sk, BQ, BK, dq, dk)
+    mask = materialize_mask_terms(terms, B, Sq, Sk, dq, dk, device=gpu)
+    want = compute_mask_kernel(mask.expand(B, H, Sq, Sk), BQ, BK, pack_partial=True)
+    same_metadata(md, want, BQ, BK)
+    m_or = oracle.mask_from_terms([t.encode() for t in terms], B, Sq, Sk, dq.cpu().numpy(), dk.cpu().numpy())
+    assert np.array_equal(m_or, mask.expand(B, 1, Sq, Sk)[:, 0].cpu().numpy())
