@@ -284,16 +284,29 @@ __global__ __launch_bounds__(256, 2) void sparse_bwd_kernel(const BwdParams p) {
     }
 
     // out = acc * out_scale; acc holds the transposed tile: lane (row l32, hh), register 4g + jj of block db is
-    // d = 32 db + 8g + 4hh + jj
-    uint16_t *orow = p.out + b * p.outs[0] + h * p.outs[1] + (int64_t)rrow * p.outs[2] + 4 * hh;
+    // d = 32 db + 8g + 4hh + jj.  A lane's 8-byte pieces would make every store instruction touch 32 rows, so the
+    // wave's 32 rows go through a private slice of the (now idle) chunk buffers, rows 16 bytes apart from the banks'
+    // period, and leave as whole rows, 16 bytes per lane.
+    __syncthreads();  // every wave is done with the chunk buffers
+    constexpr int OROW = ROWB + 16;
+    static_assert(4 * 32 * OROW <= 4 * CBUF, "the rows of the four waves fit the chunk buffers");
+    uint8_t *const ob = smem + wave * 32 * OROW;
 #pragma unroll
     for (int db = 0; db < NDB; db++)
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             const u32x2 w = {E::pack2(acc[db][4 * g] * p.out_scale, acc[db][4 * g + 1] * p.out_scale),
                              E::pack2(acc[db][4 * g + 2] * p.out_scale, acc[db][4 * g + 3] * p.out_scale)};
-            *(u32x2 *)(orow + 32 * db + 8 * g) = w;
+            *(u32x2 *)(ob + l32 * OROW + 2 * (32 * db + 8 * g + 4 * hh)) = w;
         }
+    constexpr int PPR_O = ROWB / 16;  // 16-byte pieces per row
+    uint16_t *const o0 = p.out + b * p.outs[0] + h * p.outs[1] + (int64_t)(rt * 128 + wave * 32) * p.outs[2];
+#pragma unroll
+    for (int i = 0; i < 32 * PPR_O / 64; i++) {
+        const int idx = 64 * i + lane, r = idx / PPR_O, pc = idx % PPR_O;
+        const u32x4 x = *(const u32x4 *)(ob + r * OROW + 16 * pc);
+        *(u32x4 *)(o0 + (int64_t)r * p.outs[2] + 8 * pc) = x;
+    }
 }
 
 // Per query row: Delta = sum_d dO o O, and L = lse / ln 2 (+inf for rows that attended to nothing, so that their

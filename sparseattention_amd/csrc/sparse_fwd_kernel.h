@@ -637,6 +637,36 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
             }
     };
 
+    // The same through LDS, for paths that end with every K/V stage free (no wave reads them any more, no direct load
+    // is on its way): a lane owns 8-byte pieces of its own row, which makes every store instruction touch 32 rows; a
+    // wave-private copy of its 32 rows in LDS (rows 16 bytes apart from the banks' period) read back 16 bytes per
+    // lane turns them into stores of whole rows, an eighth of the memory transactions.
+    auto store_o_rows = [&]() {
+        const float l_tot = l32 < 16 ? acc_l[0] : acc_l[1];
+        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        if (p.lse != nullptr && hh == 0)
+            p.lse[lse_off] = l_tot > 0.f ? (m_ref + __builtin_amdgcn_logf(l_tot)) * 0.69314718056f : kNegInf;
+        constexpr int OROW = ROWB + 16;
+        static_assert(NW * 32 * OROW <= 2 * NS * 64 * ROWB, "the rows of all waves fit the K/V stages");
+        uint8_t *const ob = smem + wave * 32 * OROW;
+#pragma unroll
+        for (int db = 0; db < D / 32; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const u32x2 w = {E::pack2(acc[db][4 * g] * inv, acc[db][4 * g + 1] * inv),
+                                 E::pack2(acc[db][4 * g + 2] * inv, acc[db][4 * g + 3] * inv)};
+                *(u32x2 *)(ob + l32 * OROW + 2 * (32 * db + 8 * g + 4 * hh)) = w;
+            }
+        // 64 lanes x 16 bytes = 1024 / ROWB rows per store
+        uint16_t *const o0 = p.o + b * p.os[0] + h * p.os[1] + (int64_t)(qt * (NW * 32) + wave * 32) * p.os[2];
+#pragma unroll
+        for (int i = 0; i < 32 * PPR / 64; i++) {
+            const int idx = 64 * i + lane, r = idx / PPR, pc = idx % PPR;
+            const u32x4 x = *(const u32x4 *)(ob + r * OROW + 16 * pc);
+            *(u32x4 *)(o0 + (int64_t)r * p.os[2] + 8 * pc) = x;
+        }
+    };
+
     if constexpr (PS) {
         // Persistent loop.  Per Q tile of this workgroup's row, the pipeline is
         //   two tiles ahead  its schedule entry is loaded;
@@ -958,7 +988,8 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
         }
     }
 
-    store_o();
+    if constexpr (PP) store_o();  // (the late waves of the ping-pong schedule still read their last stage)
+    else store_o_rows();
 }
 
 template <int DT, int D, int NW, int MODE, bool PK, bool PS>
