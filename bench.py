@@ -39,13 +39,13 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E peak, GB/s
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this script and scaled by
 # the readings of a 1 GiB device copy in the same run (--calibrate-copy).  The summaries with the commands
 # are profiles/sparse_fwd_kernel_causal_B8H32S4096D128.txt and profiles/mask_classify_kernels_mask_32768x32768.txt.
-TRAFFIC_FWD_CAUSAL_BYTES = 1.2835e9      # 967.7 MiB read + 256.3 MiB written
+TRAFFIC_FWD_CAUSAL_BYTES = 1.2828e9      # 967.1 MiB read + 256.3 MiB written
 TRAFFIC_CLASSIFY_1GIB_BYTES = 1.0744e9   # 1,048,622 + 327 KiB read, 256 + 45.5 KiB written
 # decode workloads (profiles/sparse_decode_kernel_B8H32Sk32768D128.txt), both kernels
 TRAFFIC_DECODE_BYTES = (4.2959e9, 1.6225e9)
 # backward of the headline workload (profiles/sparse_bwd_kernel_causal_B8H32S4096D128.txt), three passes + prepare:
-# 4256 MiB read + 778.7 MiB written
-TRAFFIC_BWD_CAUSAL_BYTES = 5.280e9
+# 4242 MiB read + 776 MiB written
+TRAFFIC_BWD_CAUSAL_BYTES = 5.262e9
 
 B, H, S, D = 8, 32, 4096, 128
 BQ, BK = 128, 32
@@ -73,15 +73,16 @@ def time_launches(fn, steps, warmup):
     events recorded on the stream the kernel is launched on (torch's current stream)."""
     import torch
 
-    for _ in range(warmup):
-        fn()
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    # a collection of the interpreter's cyclic garbage inside the timed region costs tens of milliseconds of host
-    # time, which a microsecond-scale step would report as its own
+    # A collection of the interpreter's cyclic garbage costs tens of milliseconds of host time: inside the timed region
+    # a microsecond-scale step would report it as its own, and between warm-up and timed region it lets the device
+    # fall idle, after which the next ten launches run up to 40 % slow.  So it happens before the warm-up.
     gc.collect()
     gc.disable()
     try:
+        for _ in range(warmup):
+            fn()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(steps):
@@ -361,7 +362,8 @@ def main():
                      "flop_per_launch": head["_executed_flop"]},
     }
     if not args.no_sweep:
-        vs, vw = max(5, args.steps // 2), max(2, args.warmup // 2)
+        # (a launch after an idle gap runs up to 40 % slow and the next ten settle: never fewer than 10 warm-ups)
+        vs, vw = max(20, args.steps // 2), max(10, args.warmup)
         causal = W.causal_mask(S, "cuda")
         result["variants"] = {
             name: round(forward_case(name, causal, q, k, v, vs, vw, schedule=sch, pack_partial=pk)["kernel_ms"], 4)
@@ -370,7 +372,7 @@ def main():
                                   ("persistent_schedule_packed_ms", "persistent", True))}
         del causal
         rows = [head]
-        sweep_steps, sweep_warm = max(5, args.steps // 5), max(2, args.warmup // 3)
+        sweep_steps, sweep_warm = max(20, args.steps // 2), max(10, args.warmup)
         rows.append(forward_case("dense (all True)", torch.ones(S, S, dtype=torch.bool, device="cuda"), q, k, v,
                                  sweep_steps, sweep_warm))
         for p in (0.25, 0.5, 0.75, 0.9):
@@ -382,10 +384,10 @@ def main():
         result["mask_terms"] = terms_case(max(10, args.steps // 2), max(3, args.warmup // 2))
         result["mask_classify_headline"] = classify_small_case(max(10, args.steps // 2), max(3, args.warmup // 2))
     if not args.no_backward:
-        result["backward"] = backward_case(q, k, v, max(5, args.steps // 5), max(2, args.warmup // 3))
+        result["backward"] = backward_case(q, k, v, max(10, args.steps // 5), max(5, args.warmup // 2))
     del q, k, v
     if not args.no_decode:
-        result["decode"] = decode_case(max(10, args.steps // 2), max(3, args.warmup // 2))
+        result["decode"] = decode_case(max(20, args.steps // 2), max(10, args.warmup))
     if args.calibrate_copy:
         src = torch.ones(1 << 28, dtype=torch.int32, device="cuda")  # 1 GiB read + 1 GiB written per copy
         dst = torch.empty_like(src)
