@@ -988,8 +988,8 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
         }
     }
 
-    if constexpr (PP) store_o();  // (the late waves of the ping-pong schedule still read their last stage)
-    else store_o_rows();
+    if constexpr (PP) __syncthreads();  // the late waves of the ping-pong schedule have read their last stage
+    store_o_rows();
 }
 
 template <int DT, int D, int NW, int MODE, bool PK, bool PS>
