@@ -284,6 +284,49 @@ def test_runs_on_a_side_stream(gpu):
     assert torch.equal(got, want)
 
 
+def test_calls_from_several_host_threads(gpu):
+    # four host threads, each with a stream of its own and shapes of its own (so each is the first to raise the LDS
+    # limit of some kernel variant), forward with preprocessing, lse and errors in between: the results equal the
+    # ones computed one after the other, and an error message stays with the thread that caused it
+    import threading
+
+    cases = [(1, 2, 256, 64, 64, 32), (2, 1, 512, 128, 128, 64), (1, 3, 384, 128, 128, 16), (2, 2, 256, 64, 32, 128)]
+    inputs = []
+    for i, (B, H, S, D, BQ, BK) in enumerate(cases):
+        q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=40 + i, device=gpu)
+        mask = W.random_block_mask(S, 32, 0.5, seed=50 + i, device=gpu)
+        inputs.append((q, k, v, mask, BQ, BK))
+    want = [sparse_attention(*inp, return_lse=True) for inp in inputs]
+    torch.cuda.synchronize()
+    got, errors = [None] * len(cases), []
+
+    def work(i):
+        try:
+            s = torch.cuda.Stream()
+            with torch.cuda.stream(s):
+                for _ in range(5):
+                    got[i] = sparse_attention(*inputs[i], return_lse=True)
+                    q, k, v, mask, BQ, BK = inputs[i]
+                    try:
+                        sparse_attention(q[..., :48], k[..., :48], v[..., :48], mask, BQ, BK)
+                        errors.append(f"thread {i}: head dim 48 was accepted")
+                    except _native.SparseAttnError as e:
+                        if "head dim 48" not in str(e):
+                            errors.append(f"thread {i}: foreign message {e}")
+            s.synchronize()
+        except Exception as e:  # noqa: BLE001 - reported by the assertion below
+            errors.append(f"thread {i}: {type(e).__name__} {e}")
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(len(cases))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for (o, lse), (o_w, lse_w) in zip(got, want):
+        assert torch.equal(o, o_w) and torch.equal(lse, lse_w)
+
+
 @pytest.mark.parametrize("route", ["plain", "packed+pairs", "persistent"])
 @pytest.mark.parametrize("BQ,BK", [(128, 32), (64, 64), (256, 16)])
 def test_lse_output(gpu, route, BQ, BK):
