@@ -97,17 +97,17 @@ def time_launches(fn, steps, warmup):
     return wall_ms, ev_ms
 
 
-def forward_case(name, mask2d, q, k, v, steps, warmup, schedule=None, pack_partial=None):
+def forward_case(name, mask2d, q, k, v, steps, warmup, schedule=None, pack_partial=None, block_k=BK):
     import torch
     from sparseattention_amd import compute_mask_kernel, sparse_attention
 
     me = mask2d[None, None].expand(B, H, S, S)
-    md = compute_mask_kernel(me, BQ, BK, pack_partial=pack_partial, schedule=schedule)
+    md = compute_mask_kernel(me, BQ, block_k, pack_partial=pack_partial, schedule=schedule)
     tiles_plane = int(md.unmasked_lens[0, 0].sum()) + int(md.masked_lens[0, 0].sum())
     partial_plane = int(md.masked_lens[0, 0].sum())
     frac = float(mask2d.float().mean())
-    wall_ms, ev_ms = time_launches(lambda: sparse_attention(q, k, v, me, BQ, BK, mask_metadata=md), steps, warmup)
-    executed = tiles_plane * B * H * FLOP_PER_TILE
+    wall_ms, ev_ms = time_launches(lambda: sparse_attention(q, k, v, me, BQ, block_k, mask_metadata=md), steps, warmup)
+    executed = tiles_plane * B * H * 4 * BQ * block_k * D
     useful = 4 * B * H * S * S * D * frac
     return {
         "mask": name,
@@ -370,6 +370,9 @@ def main():
             for name, sch, pk in (("pairs_schedule_packed_ms", "pairs", True), ("no_schedule_packed_ms", None, True),
                                   ("no_schedule_bool_mask_ms", None, False),
                                   ("persistent_schedule_packed_ms", "persistent", True))}
+        # the same mask tiled 128 x 64 (the same executed area; the forward consumes keys in chunks of 64 either way)
+        result["variants"]["tiles_128x64_ms"] = round(
+            forward_case("causal 128x64", causal, q, k, v, vs, vw, block_k=64)["kernel_ms"], 4)
         del causal
         rows = [head]
         sweep_steps, sweep_warm = max(20, args.steps // 2), max(10, args.warmup)
