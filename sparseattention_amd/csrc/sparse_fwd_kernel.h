@@ -348,11 +348,15 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
     struct StagePlan {
         const uint16_t *kp[EPC], *vp[EPC];  // first row of every list entry of the chunk (scalar registers)
     };
+    // first row of a list entry as an element offset: key column and row stride are both below 2^32 (the strides
+    // are checked on the host), so one 32 x 32 -> 64 bit product does
+    const uint32_t ks2 = (uint32_t)p.ks[2], vs2 = (uint32_t)p.vs[2];
+    auto row_off = [](int col, uint32_t stride) -> int64_t { return (int64_t)((uint64_t)(uint32_t)col * stride); };
     auto plan_chunk = [&](const int(&col)[EPC], StagePlan &pl) {
 #pragma unroll
         for (int j = 0; j < EPC; j++) {
-            pl.kp[j] = kbase + (int64_t)col[j] * p.ks[2];
-            pl.vp[j] = vbase + (int64_t)col[j] * p.vs[2];
+            pl.kp[j] = kbase + row_off(col[j], ks2);
+            pl.vp[j] = vbase + row_off(col[j], vs2);
         }
     };
     auto stage_piece = [&](int buf, int piece, const StagePlan &pl) {
@@ -750,8 +754,8 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
                     const uint16_t *vn = p.v + nb_ * p.vs[0] + nh_ * p.vs[1];
 #pragma unroll
                     for (int e = 0; e < EPC; e++) {
-                        pl.kp[e] = kn + (int64_t)coln[e] * p.ks[2];
-                        pl.vp[e] = vn + (int64_t)coln[e] * p.vs[2];
+                        pl.kp[e] = kn + row_off(coln[e], ks2);
+                        pl.vp[e] = vn + row_off(coln[e], vs2);
                     }
                     sp[nxt] = part != 0u || valid != ALL;
                     vl[nxt] = valid;
@@ -772,8 +776,8 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
                     if (bb == 0) ps_entries_use(t2, raw, col2, valid2, part2);
 #pragma unroll
                     for (int i = bb * per; i < (bb + 1) * per && i < 2 * EPC; i++) {
-                        if (i & 1) pl2.vp[i >> 1] = vbase + (int64_t)col2[i >> 1] * p.vs[2];
-                        else pl2.kp[i >> 1] = kbase + (int64_t)col2[i >> 1] * p.ks[2];
+                        if (i & 1) pl2.vp[i >> 1] = vbase + row_off(col2[i >> 1], vs2);
+                        else pl2.kp[i >> 1] = kbase + row_off(col2[i >> 1], ks2);
                     }
                     if (bb == nb - 1) ps_entries_read(el, t3, raw);
                 });
@@ -967,8 +971,8 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
                         if (b == 0) entries_use(t2, raw, col2, valid2, part2);
 #pragma unroll
                         for (int i = b * per; i < (b + 1) * per && i < 2 * EPC; i++) {
-                            if (i & 1) pl2.vp[i >> 1] = vbase + (int64_t)col2[i >> 1] * p.vs[2];
-                            else pl2.kp[i >> 1] = kbase + (int64_t)col2[i >> 1] * p.ks[2];
+                            if (i & 1) pl2.vp[i >> 1] = vbase + row_off(col2[i >> 1], vs2);
+                            else pl2.kp[i >> 1] = kbase + row_off(col2[i >> 1], ks2);
                         }
                         if (b == nb - 1) entries_read(t3, raw);
                     });
