@@ -76,11 +76,13 @@ def scratch_offenders(resources: dict) -> dict:
 
     Every kernel of this library keeps its state in registers.  One whose arrays the compiler could not split into
     registers (scratch memory without spilled registers: a variable index into a small array is enough) runs several
-    times slower with the same results, which no parity test would notice; so does one that spills many registers.
+    times slower with the same results, which no parity test would notice; so does one that spills many registers
+    to scratch memory (registers "spilled" without any scratch went to the other half of the register file of a
+    kernel that runs one wave per SIMD, which is no concern).
     """
     return {k: v for k, v in resources.items()
-            if (v.get("ScratchSize", 0) and not v.get("VGPRsSpill", 0)) or v.get("DynamicStack", 0)
-            or v.get("VGPRsSpill", 0) > MAX_SPILLED_VGPRS}
+            if v.get("DynamicStack", 0)
+            or (v.get("ScratchSize", 0) and not 0 < v.get("VGPRsSpill", 0) <= MAX_SPILLED_VGPRS)}
 
 
 def _run(cmd):

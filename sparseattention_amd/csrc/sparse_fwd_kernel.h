@@ -239,52 +239,47 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
     // The Q tile's list (FULL entries, then PARTIAL entries) as first key columns, copied to LDS once:
     // loads issued after the first barrier cannot use the scalar cache, and a vector load of an index in
     // front of every chunk would put a full memory round trip on the critical path.
-    const bool list_in_lds = !PS && NE <= kListCap;
+    // Every entry carries its kind in the top bits, and the list is padded with ABSENT entries to whole chunks, so
+    // that a chunk's entries say by themselves which of them exist and which are PARTIAL:
+    //   bits 0..29 first key column, bit 30 PARTIAL, bit 31 ABSENT (column 0: its scores are discarded).
+    constexpr int kPartialBit = 1 << 30;
+    constexpr int kAbsent = (int)0x80000000u;
+    const int list_cnt = MODE == 2 ? NE : (NE + EPC - 1) / EPC * EPC;
+    const bool list_in_lds = !PS && list_cnt <= kListCap;
+    auto tagged_entry = [&](int e) -> int {  // from global memory
+        if (e >= NE) return kAbsent;
+        const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
+        return (MODE == 2 ? (idx << p.lbk) : (idx << LBKC)) | (e >= F ? kPartialBit : 0);
+    };
     if (list_in_lds) {
-        for (int e = tid; e < NE; e += NW * 64) {
-            const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
-            ent[e] = MODE == 2 ? (idx << p.lbk) : (idx << LBKC);
-        }
+        for (int e = tid; e < list_cnt; e += NW * 64) ent[e] = tagged_entry(e);
     }
     // First key column of every list entry in chunk t (t < T), plus which entries exist / are partial, in two
     // steps: entries_read issues the reads of the list (the values are the same in all lanes), entries_use turns
     // them into scalars.  The main loop reads the entries of a chunk one iteration before it needs them, so
     // that no wave waits for the list.
     auto entry_read = [&](int e) -> int {
-        if (list_in_lds) return ent[e];
-        const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
-        return MODE == 2 ? (idx << p.lbk) : (idx << LBKC);
+        if (__builtin_expect(list_in_lds, 1)) return ent[e];
+        return tagged_entry(e);
     };
     auto entries_read = [&](int t, int(&raw)[EPC]) {
         if constexpr (MODE == 2) {
             raw[0] = entry_read(t >> (p.lbk - 6));
         } else {
 #pragma unroll
-            for (int j = 0; j < EPC; j++) {
-                const int e = t * EPC + j;
-                raw[j] = entry_read(e < NE ? e : t * EPC);  // absent entries re-read the chunk's first one;
-            }                                                // their scores are discarded
+            for (int j = 0; j < EPC; j++) raw[j] = entry_read(t * EPC + j);
         }
     };
     auto entries_use = [&](int t, const int(&raw)[EPC], int(&col)[EPC], unsigned &valid, unsigned &part) {
         valid = 0u;
         part = 0u;
-        if constexpr (MODE == 2) {
-            const int sh = p.lbk - 6;
-            const int e = t >> sh, sub = t & ((1 << sh) - 1);
-            col[0] = __builtin_amdgcn_readfirstlane(raw[0]) + (sub << 6);
-            valid = 1u;
-            part = e >= F ? 1u : 0u;
-        } else {
 #pragma unroll
-            for (int j = 0; j < EPC; j++) {
-                const int e = t * EPC + j;
-                col[j] = __builtin_amdgcn_readfirstlane(raw[j]);
-                if (e < NE) {
-                    valid |= 1u << j;
-                    if (e >= F) part |= 1u << j;
-                }
-            }
+        for (int j = 0; j < EPC; j++) {
+            const int v = __builtin_amdgcn_readfirstlane(raw[j]);
+            col[j] = v & (kPartialBit - 1);
+            if constexpr (MODE == 2) col[j] += (t & ((1 << (p.lbk - 6)) - 1)) << 6;
+            if (v >= 0) valid |= 1u << j;
+            if (v & kPartialBit) part |= 1u << j;
         }
     };
     auto chunk_entries = [&](int t, int(&col)[EPC], unsigned &valid, unsigned &part) {
@@ -297,7 +292,6 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
     //   bits 0..29 first key column, bit 30 PARTIAL, bit 31 ABSENT.
     constexpr int NT = NW * 64;
     constexpr int PER = kPsListCap / NT;  // list entries per thread
-    constexpr int kPartialBit = 1 << 30;
     const int lbk_rt = MODE == 2 ? p.lbk : LBKC;
     auto ps_list_issue = [&](int b_, int h_, int qt_, int F_, int P_, int(&lr)[PER]) {  // indices -> registers
         const int32_t *f_ = p.full_ids + b_ * p.fis[0] + h_ * p.fis[1] + qt_ * p.fis[2];
@@ -317,7 +311,7 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
 #pragma unroll
         for (int i = 0; i < PER; i++) {
             const int e = tid + NT * i;
-            if (e < cnt) dst[e] = e >= ne ? (int)0x80000000u : ((lr[i] << lbk_rt) | (e >= F_ ? kPartialBit : 0));
+            if (e < cnt) dst[e] = e >= ne ? kAbsent : ((lr[i] << lbk_rt) | (e >= F_ ? kPartialBit : 0));
         }
     };
     auto ps_entries_read = [&](const int *el, int t, int(&raw)[EPC]) {

@@ -215,6 +215,7 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
     }
     if (o_strides[2] == 0 || (B > 1 && o_strides[0] == 0) || (H > 1 && o_strides[1] == 0))
         return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd: o must not alias itself (zero stride)");
+    if (Sk >= (1 << 30)) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: Sk %d (supported: below 2^30)", Sk);
     // (the kernels form row offsets of K and V from 32-bit factors)
     if (k_strides[2] < 0 || v_strides[2] < 0 || k_strides[2] >= (1 << 24) || v_strides[2] >= (1 << 24))
         return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: row strides of k and v must lie in [0, 2^24) elements (%lld, %lld)",

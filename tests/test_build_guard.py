@@ -44,3 +44,5 @@ def test_arrays_in_scratch_and_heavy_spills_are_refused():
     res["_Z6kernelILi1EEv1P"]["VGPRsSpill"] = MAX_SPILLED_VGPRS + 1
     assert list(scratch_offenders(res)) == ["_Z6kernelILi0EEv1P", "_Z6kernelILi1EEv1P"]
     assert scratch_offenders({"k": {"VGPRs": 10, "ScratchSize": 0, "DynamicStack": 1}}) == {"k": {"VGPRs": 10, "ScratchSize": 0, "DynamicStack": 1}}
+    # registers moved to the other half of the register file (no scratch) are no concern
+    assert scratch_offenders({"k": {"VGPRs": 256, "AGPRs": 200, "ScratchSize": 0, "VGPRsSpill": 32}}) == {}
