@@ -47,6 +47,8 @@ TRAFFIC_DECODE_BYTES = (4.2959e9, 1.6225e9)
 # 4242 MiB read + 776 MiB written
 TRAFFIC_BWD_CAUSAL_BYTES = 5.262e9
 
+SETTLE_LAUNCHES = 30
+
 B, H, S, D = 8, 32, 4096, 128
 BQ, BK = 128, 32
 FLOP_PER_TILE = 4 * BQ * BK * D
@@ -81,6 +83,10 @@ def time_launches(fn, steps, warmup):
     gc.collect()
     gc.disable()
     try:
+        # the device settles over its first ten to twenty launches after an idle gap: with a short warm-up, further
+        # untimed launches go in front of it
+        for _ in range(max(0, SETTLE_LAUNCHES - warmup)):
+            fn()
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
