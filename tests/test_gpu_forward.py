@@ -394,3 +394,24 @@ def test_head_dim_256_limits_and_long_rows(gpu):
     mask = W.causal_mask(S, gpu)
     o = sparse_attention(q, k, v, mask, 128, 32)
     assert (o.float() - sdpa32(q, k, v, mask)).abs().max() <= TOL
+
+
+@pytest.mark.parametrize("BK", [16, 32, 64])
+def test_lists_longer_than_the_lds_copy(gpu, BK):
+    # more list entries per Q tile than the kernel keeps in LDS (2048): the entries are then read from global memory
+    # chunk by chunk; FULL and PARTIAL entries, an odd count, with and without packed tiles
+    B, H, Sq, D = 1, 2, 128, 64
+    Sk = BK * 2048 + 5 * BK * (64 // BK if BK < 64 else 1) + BK * 3
+    Sk = (Sk + 63) // 64 * 64
+    q, _, _ = W.qkv(B, H, Sq, D, torch.bfloat16, seed=61, device=gpu)
+    _, k, v = W.qkv(B, H, Sk, D, torch.bfloat16, seed=62, device=gpu)
+    mask = torch.ones(Sq, Sk, dtype=torch.bool, device=gpu)
+    mask[:, 1000:1000 + 3 * BK] = torch.rand(Sq, 3 * BK, generator=torch.Generator().manual_seed(63)).to(gpu) < 0.5
+    mask[:, 5000:5000 + BK] = False
+    me = mask[None, None].expand(B, H, Sq, Sk)
+    want = sdpa32(q, k, v, mask)
+    for pack in (False, True):
+        md = compute_mask_kernel(me, 128, BK, pack_partial=pack)
+        assert int(md.unmasked_lens[0, 0, 0] + md.masked_lens[0, 0, 0]) > 2048
+        o = sparse_attention(q, k, v, me, 128, BK, mask_metadata=md)
+        assert (o.float() - want).abs().max() <= TOL
