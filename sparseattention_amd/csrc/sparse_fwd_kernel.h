@@ -31,6 +31,14 @@ namespace sa {
 
 namespace {
 
+// Issue priority of a wave by phase of its chunk (s_setprio; 0 outside the two phases).  The two waves that share
+// a SIMD both want the matrix pipe most of the time; served alternately they leave their MFMA phases together and
+// then do their vector and scalar work together, with the pipe idle.  Letting the wave in its P.V phase (MFMAs
+// with exponentials between them) go ahead of one in its S phase (MFMAs only), and either ahead of the
+// bookkeeping between chunks, keeps them apart: 3 % on the causal and 2 % on the dense workload at D = 128.
+constexpr int kPrioS = 1;
+constexpr int kPrioPV = 2;
+
 // "At most n vector-memory operations of this wave still in flight", n a small run-time value.
 __device__ __forceinline__ void wait_vm_at_most(int n, int step) {
     if (n <= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -502,6 +510,8 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
 #pragma unroll
         for (int c = 0; c < kPfS; c++) k_read(c);
         __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_setprio(kPrioS);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int c = 0; c < NC; c++) {
             s[1] = E::mfma(kf1[c], qf[c], c == 0 ? neg_m : s[1]);
@@ -513,6 +523,8 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
             }
             __builtin_amdgcn_sched_barrier(0);
         }
+        __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_sched_barrier(0);
     };
     // P.V phase: mask, online softmax, O^T += V^T . P^T.  between(b, NB) is called once per MFMA bundle b of NB;
     // the main loop uses it to spread scalar bookkeeping over the phase, where it hides behind the MFMAs.
@@ -592,6 +604,8 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
         for (int b = 0; b < kPfV; b++) v_read(b);
         p_values(0, 0, 8);
         __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_setprio(kPrioPV);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int b = 0; b < NB; b++) {
             const int kc = b / BPK;
@@ -607,6 +621,8 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
             between(b, NB);
             __builtin_amdgcn_sched_barrier(0);
         }
+        __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_sched_barrier(0);
     };
 
     // Makes the compiler account for a completed vector-memory load here (it emits its own wait, which
