@@ -17,6 +17,29 @@ def _kernel_ready(t: torch.Tensor) -> torch.Tensor:
     return t if ok else t.contiguous()
 
 
+_KERNEL_BLOCK_Q = (128, 64, 32, 256)  # in order of preference when the caller's size is not one of them
+
+
+def kernel_tiles(Sq: int, Sk: int, D: int, BLOCK_Q: int, BLOCK_K: int):
+    """The tile sizes the forward runs a request for ``BLOCK_Q`` x ``BLOCK_K`` tiles with: the same pair when the
+    kernels tile by it (BLOCK_Q 32/64/128/256 — 64/128 at head dim 256 —, BLOCK_K a power of two >= 16), else the
+    nearest pair they have that divides Sq and Sk, or None when there is none.  The reference takes any sizes its
+    compiler accepts (sparse_attn_kernel.py:149-185); the result does not depend on them."""
+    BLOCK_Q, BLOCK_K = int(BLOCK_Q), int(BLOCK_K)
+    ok_k = BLOCK_K >= 16 and BLOCK_K & (BLOCK_K - 1) == 0 and Sk % BLOCK_K == 0
+    if Sq < 32:  # the few-rows kernels: one Q tile of all rows, KV tiles of 32 keys or more
+        if ok_k and BLOCK_K >= 32:
+            return Sq, BLOCK_K
+        return next(((Sq, bk) for bk in (32, 64) if Sk % bk == 0), None)
+    ok_q = [b for b in _KERNEL_BLOCK_Q if Sq % b == 0 and (D != 256 or b in (64, 128))]
+    if not ok_q:
+        return None
+    bq = BLOCK_Q if BLOCK_Q in ok_q else ok_q[0]
+    if ok_k:
+        return bq, BLOCK_K
+    return next(((bq, bk) for bk in (32, 64, 16) if Sk % bk == 0), None)
+
+
 def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor | None, BLOCK_Q, BLOCK_K,
                      mask_metadata: MaskMetadata | None = None, *, return_lse: bool = False):
     """softmax(q kᵀ / sqrt(D) + (mask ? 0 : -inf)) v, skipping KV tiles the mask empties.
@@ -43,14 +66,33 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
         raise TypeError(f"q, k, v must share dtype bfloat16 or float16 (got {q.dtype}, {k.dtype}, {v.dtype})")
     if mask is None and getattr(mask_metadata, "packed_masks", None) is None:
         raise ValueError("sparse_attention without a mask tensor needs mask_metadata with packed_masks")
+    if mask is not None:
+        mask = mask.expand(B, H, Sq, Sk)
+    BLOCK_Q, BLOCK_K = int(BLOCK_Q), int(BLOCK_K)
+    tiles = kernel_tiles(Sq, Sk, D, BLOCK_Q, BLOCK_K)
+    if tiles != (BLOCK_Q, BLOCK_K):
+        # Tile sizes the kernels do not tile by.  They only say how the mask is cut up, not what is computed, so the
+        # mask is classified again at sizes the kernels have; the lists are kept on the caller's metadata.
+        # what the reference asserts (mask_utils.py:89-90)
+        assert Sq % BLOCK_Q == 0 and Sk % BLOCK_K == 0, \
+            f"Sq={Sq} / Sk={Sk} must be multiples of BLOCK_Q={BLOCK_Q} / BLOCK_K={BLOCK_K}"
+        if tiles is None or mask is None:
+            raise ValueError(f"sparse_attention: no kernel tiles for BLOCK_Q={BLOCK_Q}, BLOCK_K={BLOCK_K} at Sq={Sq}, "
+                             f"Sk={Sk}, D={D}" + ("" if tiles is None else " without a mask tensor to classify again"))
+        again = getattr(mask_metadata, "_retiled", None)
+        if again is None or again[0] != (tiles, mask.data_ptr(), tuple(mask.stride()), mask._version):
+            again = ((tiles, mask.data_ptr(), tuple(mask.stride()), mask._version),
+                     compute_mask_kernel(mask, *tiles, pack_partial=None if Sq >= 32 else False))
+            if mask_metadata is not None:
+                mask_metadata._retiled = again
+        BLOCK_Q, BLOCK_K = tiles
+        mask_metadata = again[1]
+
     if (Sq == BLOCK_Q and Sq < 32 and BLOCK_K >= 32 and getattr(mask_metadata, "packed_masks", None) is None
             and getattr(mask_metadata, "schedule", None) is None):
         # one Q tile of fewer rows than the forward kernels tile by: the split-KV kernels
         return sparse_attention_decode(q, k, v, mask, BLOCK_K, mask_metadata, return_lse=return_lse)
     sm_scale = D ** (-0.5) * 1 / math.log(2)  # exp2 replaces exp (sparse_attn_kernel.py:152)
-
-    if mask is not None:
-        mask = mask.expand(B, H, Sq, Sk)
 
     if mask_metadata is None:
         mask_metadata = compute_mask_kernel(mask, BLOCK_Q, BLOCK_K)

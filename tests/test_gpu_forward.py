@@ -175,10 +175,42 @@ def test_wrapper_errors(gpu):
     with pytest.raises(_native.SparseAttnError, match="head dim"):
         sparse_attention(qb, qb, qb, m, 128, 32)
     qb = torch.zeros(1, 1, 128, 128, dtype=torch.bfloat16, device=gpu)
-    with pytest.raises(_native.SparseAttnError, match="BLOCK_Q"):
-        sparse_attention(qb, qb, qb, m, 16, 32)
     with pytest.raises(AssertionError):
         sparse_attention(qb, qb, qb, m, 128, 48)
+    with pytest.raises(ValueError, match="no kernel tiles"):  # 40 rows: more than the few-rows kernels take, no tile fits
+        sparse_attention(qb[:, :, :40], qb, qb, m[:40], 8, 32)
+    # tiles the kernels do not have are refused at the C ABI and need a mask tensor in the wrapper
+    md = compute_mask_kernel(m[None, None], 16, 32)
+    with pytest.raises(ValueError, match="without a mask tensor"):
+        sparse_attention(qb, qb, qb, None, 16, 32, mask_metadata=md)
+
+
+@pytest.mark.parametrize("Sq,D,BQ,BK", [(256, 128, 16, 32), (256, 128, 16, 8), (1024, 64, 512, 4), (256, 256, 32, 32),
+                                         (256, 256, 256, 64), (16, 128, 8, 16), (24, 64, 24, 8), (96, 128, 48, 32)])
+def test_tile_sizes_the_kernels_do_not_have(gpu, Sq, D, BQ, BK):
+    """Any tile sizes that divide the mask work, as in the reference: the wrapper classifies the mask again at sizes the
+    kernels tile by, once per metadata object and mask."""
+    from sparseattention_amd.sparse_attn_kernel import kernel_tiles
+    B, H, Sk = 2, 2, 512
+    q, k, v = W.qkv(B, H, Sq, D, torch.bfloat16, seed=Sq + BQ, device=gpu, Sk=Sk)
+    mask = (torch.rand(B, 1, Sq, Sk, generator=torch.Generator().manual_seed(BK)) < 0.6).to(gpu)
+    mask[..., :Sq // 2, Sk // 2:] = False
+    mask[..., 0] = True
+    tiles = kernel_tiles(Sq, Sk, D, BQ, BK)
+    assert tiles is not None and tiles != (BQ, BK) and Sq % tiles[0] == 0 and Sk % tiles[1] == 0
+    want = sdpa32(q, k, v, mask)
+    o = sparse_attention(q, k, v, mask, BQ, BK)
+    assert (o.float() - want).abs().max() <= TOL
+    assert torch.equal(o, sparse_attention(q, k, v, mask, *tiles))
+    # with the caller's metadata at its own tile sizes: classified again once, then reused
+    md = compute_mask_kernel(mask.expand(B, H, Sq, Sk), BQ, BK)
+    assert torch.equal(o, sparse_attention(q, k, v, mask, BQ, BK, mask_metadata=md))
+    again = md._retiled
+    assert torch.equal(o, sparse_attention(q, k, v, mask, BQ, BK, mask_metadata=md)) and md._retiled is again
+    mask[..., 1] = ~mask[..., 1]  # the mask changed in place: classified anew
+    o2 = sparse_attention(q, k, v, mask, BQ, BK, mask_metadata=md)
+    assert md._retiled is not again
+    assert (o2.float() - sdpa32(q, k, v, mask)).abs().max() <= TOL
 
 
 @pytest.mark.parametrize("name", golden_io.names())
@@ -385,9 +417,17 @@ def test_head_dim_256(gpu, BQ, BK, dtype):
 def test_head_dim_256_limits_and_long_rows(gpu):
     qb = torch.zeros(1, 1, 256, 256, dtype=torch.bfloat16, device=gpu)
     m = torch.ones(256, 256, dtype=torch.bool, device=gpu)
-    for BQ in (32, 256):
-        with pytest.raises(_native.SparseAttnError, match="head dim 256"):
-            sparse_attention(qb, qb, qb, m, BQ, 32)
+    lib = _native.load()
+    md = compute_mask_kernel(m[None, None], 32, 32, pack_partial=False)
+    S = _native.strides
+    me = m[None, None]
+    rc = lib.sa_sparse_attention_fwd(
+        qb.data_ptr(), S(qb.stride()), qb.data_ptr(), S(qb.stride()), qb.data_ptr(), S(qb.stride()),
+        torch.empty_like(qb).data_ptr(), S(qb.stride()), me.data_ptr(), S(me.stride()),
+        md.unmasked_kv_ids.data_ptr(), S(md.unmasked_kv_ids.stride()), md.unmasked_lens.data_ptr(),
+        S(md.unmasked_lens.stride()), md.masked_kv_ids.data_ptr(), S(md.masked_kv_ids.stride()),
+        md.masked_lens.data_ptr(), S(md.masked_lens.stride()), 1, 1, 256, 256, 256, 32, 32, 0, 0.09, None)
+    assert rc == _native.SA_ERR_UNSUPPORTED and "head dim 256" in lib.sa_last_error().decode()
     # causal, 4096 keys: long lists, every plane against fp32 SDPA
     B, H, S, D = 1, 4, 4096, 256
     q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=77, device=gpu)
