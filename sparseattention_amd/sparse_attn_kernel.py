@@ -17,6 +17,17 @@ def _kernel_ready(t: torch.Tensor) -> torch.Tensor:
     return t if ok else t.contiguous()
 
 
+def _kernel_head_dim(D: int, sizes) -> int:
+    """The head dim the kernels run a request for ``D`` with: the smallest of ``sizes`` that holds it (q, k, v are then
+    padded with zero columns, which change neither the scores nor the first D columns of the result; the softmax scale
+    stays that of D).  A D beyond all of them is passed on, for the library to refuse."""
+    return next((s for s in sizes if D <= s), D)
+
+
+def _pad_head_dim(t: torch.Tensor, Dk: int) -> torch.Tensor:
+    return t if t.shape[-1] == Dk else torch.nn.functional.pad(t, (0, Dk - t.shape[-1]))
+
+
 _KERNEL_BLOCK_Q = (128, 64, 32, 256)  # in order of preference when the caller's size is not one of them
 
 
@@ -119,7 +130,8 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
     if sched is not None and (sched.dtype != torch.int32 or sched.device != q.device or not sched.is_contiguous()):
         raise ValueError("mask_metadata.schedule: expected a contiguous int32 tensor on q's device")
 
-    qc, kc, vc = _kernel_ready(q), _kernel_ready(k), _kernel_ready(v)
+    Dk = _kernel_head_dim(D, (64, 128, 256))
+    qc, kc, vc = (_kernel_ready(_pad_head_dim(t, Dk)) for t in (q, k, v))
     o = torch.empty_like(qc)
     lib = _native.load()
     S = _native.strides
@@ -129,7 +141,7 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
                   mask.data_ptr() if mask is not None else None, S(mask.stride()) if mask is not None else None,
                   fid.data_ptr(), S(fid.stride()), fl.data_ptr(), S(fl.stride()),
                   pid.data_ptr(), S(pid.stride()), pl.data_ptr(), S(pl.stride()))
-        tail = (B, H, Sq, Sk, D, int(BLOCK_Q), int(BLOCK_K), _DTYPES[q.dtype], sm_scale,
+        tail = (B, H, Sq, Sk, Dk, int(BLOCK_Q), int(BLOCK_K), _DTYPES[q.dtype], sm_scale,
                 torch.cuda.current_stream(q.device).cuda_stream)
         sched = getattr(mask_metadata, "schedule", None)
         lse = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device) if return_lse else None
@@ -144,6 +156,8 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
         else:
             rc = lib.sa_sparse_attention_fwd(*common, *tail)
     _native.check(rc)
+    if Dk != D:
+        o = o[..., :D].contiguous()
     return (o, lse) if return_lse else o
 
 
@@ -182,14 +196,15 @@ def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, m
     assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
     if mask.device != q.device:
         raise ValueError("mask must be on the same device as q")
-    qc, kc, vc = _kernel_ready(q), _kernel_ready(k), _kernel_ready(v)
+    Dk = _kernel_head_dim(D, (64, 128))
+    qc, kc, vc = (_kernel_ready(_pad_head_dim(t, Dk)) for t in (q, k, v))
     o = torch.empty_like(qc)
     lib = _native.load()
     S = _native.strides
     with torch.cuda.device(q.device):
         if num_splits == 0:
             num_splits = lib.sa_decode_num_splits(B, H, Sq, Sk, int(BLOCK_K))
-        ws_bytes = lib.sa_decode_workspace_bytes(B, H, Sq, D, int(num_splits))
+        ws_bytes = lib.sa_decode_workspace_bytes(B, H, Sq, Dk, int(num_splits))
         ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=q.device) if ws_bytes else None
         lse = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device) if return_lse else None
         rc = lib.sa_sparse_attention_decode(
@@ -197,11 +212,13 @@ def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, m
             o.data_ptr(), S(o.stride()), mask.data_ptr(), S(mask.stride()),
             fid.data_ptr(), S(fid.stride()), fl.data_ptr(), S(fl.stride()),
             pid.data_ptr(), S(pid.stride()), pl.data_ptr(), S(pl.stride()),
-            B, H, Sq, Sk, D, int(BLOCK_K), _DTYPES[q.dtype], sm_scale, int(num_splits),
+            B, H, Sq, Sk, Dk, int(BLOCK_K), _DTYPES[q.dtype], sm_scale, int(num_splits),
             ws.data_ptr() if ws is not None else None, ws_bytes,
             lse.data_ptr() if lse is not None else None, S(lse.stride()) if lse is not None else None,
             torch.cuda.current_stream(q.device).cuda_stream)
     _native.check(rc)
+    if Dk != D:
+        o = o[..., :D].contiguous()
     return (o, lse) if return_lse else o
 
 
@@ -275,7 +292,8 @@ def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor
             raise ValueError("sparse_attention_backward needs the mask or a BackwardMetadata with packed tiles")
         bwd_metadata = compute_backward_metadata(mask)
     sm_scale = D ** (-0.5) * 1 / math.log(2)
-    qc, kc, vc, oc, doc = (_kernel_ready(t) for t in (q, k, v, o, do))
+    Dk = _kernel_head_dim(D, (64, 128))
+    qc, kc, vc, oc, doc = (_kernel_ready(_pad_head_dim(t, Dk)) for t in (q, k, v, o, do))
     dq, dk, dv = torch.empty_like(qc), torch.empty_like(kc), torch.empty_like(vc)
     lib = _native.load()
     S = _native.strides
@@ -307,8 +325,10 @@ def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor
             mask.data_ptr() if mask is not None else None, S(mask.stride()) if mask is not None else None,
             mt.data_ptr() if mt is not None else None, S(mt.stride()) if mt is not None else None,
             *packs, *lists, ws.data_ptr(), ws_bytes,
-            B, H, Sq, Sk, D, _DTYPES[q.dtype], sm_scale, torch.cuda.current_stream(q.device).cuda_stream)
+            B, H, Sq, Sk, Dk, _DTYPES[q.dtype], sm_scale, torch.cuda.current_stream(q.device).cuda_stream)
     _native.check(rc)
+    if Dk != D:
+        dq, dk, dv = (t[..., :D].contiguous() for t in (dq, dk, dv))
     return dq, dk, dv
 
 

@@ -171,7 +171,7 @@ def test_wrapper_errors(gpu):
     m = torch.ones(128, 128, dtype=torch.bool, device=gpu)
     with pytest.raises(TypeError):
         sparse_attention(q, q, q, m, 128, 32)  # fp32 has no kernel
-    qb = torch.zeros(1, 1, 128, 96, dtype=torch.bfloat16, device=gpu)
+    qb = torch.zeros(1, 1, 128, 512, dtype=torch.bfloat16, device=gpu)
     with pytest.raises(_native.SparseAttnError, match="head dim"):
         sparse_attention(qb, qb, qb, m, 128, 32)
     qb = torch.zeros(1, 1, 128, 128, dtype=torch.bfloat16, device=gpu)
@@ -340,10 +340,11 @@ def test_calls_from_several_host_threads(gpu):
                     got[i] = sparse_attention(*inputs[i], return_lse=True)
                     q, k, v, mask, BQ, BK = inputs[i]
                     try:
-                        sparse_attention(q[..., :48], k[..., :48], v[..., :48], mask, BQ, BK)
-                        errors.append(f"thread {i}: head dim 48 was accepted")
+                        wide = 264 + 8 * i  # beyond every kernel, and different in every thread
+                        sparse_attention(*(t.repeat(1, 1, 1, 5)[..., :wide] for t in (q, k, v)), mask, BQ, BK)
+                        errors.append(f"thread {i}: head dim {wide} was accepted")
                     except _native.SparseAttnError as e:
-                        if "head dim 48" not in str(e):
+                        if f"head dim {wide}" not in str(e):
                             errors.append(f"thread {i}: foreign message {e}")
             s.synchronize()
         except Exception as e:  # noqa: BLE001 - reported by the assertion below
