@@ -77,10 +77,21 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
         raise TypeError(f"q, k, v must share dtype bfloat16 or float16 (got {q.dtype}, {k.dtype}, {v.dtype})")
     if mask is None and getattr(mask_metadata, "packed_masks", None) is None:
         raise ValueError("sparse_attention without a mask tensor needs mask_metadata with packed_masks")
+    mask_given = mask
     if mask is not None:
         mask = mask.expand(B, H, Sq, Sk)
     BLOCK_Q, BLOCK_K = int(BLOCK_Q), int(BLOCK_K)
     tiles = kernel_tiles(Sq, Sk, D, BLOCK_Q, BLOCK_K)
+    if tiles is None and mask is not None and Sq > 32 and Sq % BLOCK_Q == 0 and Sk % BLOCK_K == 0:
+        # More than 32 query rows, not a multiple of 32 (48, 80, ...): zero rows are added to q and all-False rows to
+        # the mask, and their (zero) output rows dropped again.  Nothing is kept between calls on this path.
+        pad = -Sq % 32
+        m = mask_given if mask_given.dim() >= 2 else mask_given[None]
+        m = torch.nn.functional.pad(m.expand(*m.shape[:-2], Sq, Sk), (0, 0, 0, pad), value=False)
+        out = sparse_attention(torch.nn.functional.pad(q, (0, 0, 0, pad)), k, v, m,
+                               *kernel_tiles(Sq + pad, Sk, D, BLOCK_Q, BLOCK_K), return_lse=return_lse)
+        return (out[0][:, :, :Sq].contiguous(), out[1][:, :, :Sq].contiguous()) if return_lse \
+            else out[:, :, :Sq].contiguous()
     if tiles != (BLOCK_Q, BLOCK_K):
         # Tile sizes the kernels do not tile by.  They only say how the mask is cut up, not what is computed, so the
         # mask is classified again at sizes the kernels have; the lists are kept on the caller's metadata.

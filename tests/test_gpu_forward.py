@@ -177,8 +177,6 @@ def test_wrapper_errors(gpu):
     qb = torch.zeros(1, 1, 128, 128, dtype=torch.bfloat16, device=gpu)
     with pytest.raises(AssertionError):
         sparse_attention(qb, qb, qb, m, 128, 48)
-    with pytest.raises(ValueError, match="no kernel tiles"):  # 40 rows: more than the few-rows kernels take, no tile fits
-        sparse_attention(qb[:, :, :40], qb, qb, m[:40], 8, 32)
     # tiles the kernels do not have are refused at the C ABI and need a mask tensor in the wrapper
     md = compute_mask_kernel(m[None, None], 16, 32)
     with pytest.raises(ValueError, match="without a mask tensor"):
@@ -211,6 +209,20 @@ def test_tile_sizes_the_kernels_do_not_have(gpu, Sq, D, BQ, BK):
     o2 = sparse_attention(q, k, v, mask, BQ, BK, mask_metadata=md)
     assert md._retiled is not again
     assert (o2.float() - sdpa32(q, k, v, mask)).abs().max() <= TOL
+
+
+@pytest.mark.parametrize("Sq,D,BQ,BK", [(48, 128, 16, 16), (80, 64, 16, 32), (40, 128, 8, 8), (33, 32, 33, 64)])
+def test_row_counts_no_kernel_tile_divides(gpu, Sq, D, BQ, BK):
+    """More than 32 query rows, not a multiple of 32: the wrapper pads q and the mask with rows that attend to nothing."""
+    B, H, Sk = 2, 2, 256
+    q, k, v = W.qkv(B, H, Sq, D, torch.bfloat16, seed=Sq, device=gpu, Sk=Sk)
+    for mask in ((torch.rand(Sq, Sk, generator=torch.Generator().manual_seed(BQ)) < 0.5).to(gpu),
+                 (torch.rand(B, 1, 1, Sk, generator=torch.Generator().manual_seed(BK)) < 0.5).to(gpu)):
+        mask[..., 0] = True
+        o, lse = sparse_attention(q, k, v, mask, BQ, BK, return_lse=True)
+        assert o.shape == q.shape and lse.shape == (B, H, Sq)
+        assert (o.float() - sdpa32(q, k, v, mask)).abs().max() <= TOL
+        assert torch.equal(o, sparse_attention(q, k, v, mask, BQ, BK))
 
 
 @pytest.mark.parametrize("name", golden_io.names())
