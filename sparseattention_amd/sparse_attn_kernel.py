@@ -28,6 +28,17 @@ def _pad_head_dim(t: torch.Tensor, Dk: int) -> torch.Tensor:
     return t if t.shape[-1] == Dk else torch.nn.functional.pad(t, (0, Dk - t.shape[-1]))
 
 
+def _pad_mask(mask: torch.Tensor, q_multiple: int, k_multiple: int) -> torch.Tensor:
+    """``mask`` [B,H,Sq,Sk] with all-False rows and columns added up to multiples of the two numbers; only the
+    distinct planes of a broadcast view are copied."""
+    B, H, Sq, Sk = mask.shape
+    if Sq % q_multiple == 0 and Sk % k_multiple == 0:
+        return mask
+    distinct = mask[: 1 if mask.stride(0) == 0 else B, : 1 if mask.stride(1) == 0 else H]
+    padded = torch.nn.functional.pad(distinct, (0, -Sk % k_multiple, 0, -Sq % q_multiple), value=False)
+    return padded.expand(B, H, *padded.shape[2:])
+
+
 _KERNEL_BLOCK_Q = (128, 64, 32, 256)  # in order of preference when the caller's size is not one of them
 
 
@@ -77,7 +88,6 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
         raise TypeError(f"q, k, v must share dtype bfloat16 or float16 (got {q.dtype}, {k.dtype}, {v.dtype})")
     if mask is None and getattr(mask_metadata, "packed_masks", None) is None:
         raise ValueError("sparse_attention without a mask tensor needs mask_metadata with packed_masks")
-    mask_given = mask
     if mask is not None:
         mask = mask.expand(B, H, Sq, Sk)
     BLOCK_Q, BLOCK_K = int(BLOCK_Q), int(BLOCK_K)
@@ -85,13 +95,12 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
     if tiles is None and mask is not None and Sq > 32 and Sq % BLOCK_Q == 0 and Sk % BLOCK_K == 0:
         # More than 32 query rows, not a multiple of 32 (48, 80, ...): zero rows are added to q and all-False rows to
         # the mask, and their (zero) output rows dropped again.  Nothing is kept between calls on this path.
-        pad = -Sq % 32
-        m = mask_given if mask_given.dim() >= 2 else mask_given[None]
-        m = torch.nn.functional.pad(m.expand(*m.shape[:-2], Sq, Sk), (0, 0, 0, pad), value=False)
-        out = sparse_attention(torch.nn.functional.pad(q, (0, 0, 0, pad)), k, v, m,
-                               *kernel_tiles(Sq + pad, Sk, D, BLOCK_Q, BLOCK_K), return_lse=return_lse)
-        return (out[0][:, :, :Sq].contiguous(), out[1][:, :, :Sq].contiguous()) if return_lse \
-            else out[:, :, :Sq].contiguous()
+        padded_tiles = kernel_tiles(Sq + -Sq % 32, Sk, D, BLOCK_Q, BLOCK_K)
+        if padded_tiles is not None:
+            out = sparse_attention(torch.nn.functional.pad(q, (0, 0, 0, -Sq % 32)), k, v, _pad_mask(mask, 32, 1),
+                                   *padded_tiles, return_lse=return_lse)
+            return (out[0][:, :, :Sq].contiguous(), out[1][:, :, :Sq].contiguous()) if return_lse \
+                else out[:, :, :Sq].contiguous()
     if tiles != (BLOCK_Q, BLOCK_K):
         # Tile sizes the kernels do not tile by.  They only say how the mask is cut up, not what is computed, so the
         # mask is classified again at sizes the kernels have; the lists are kept on the caller's metadata.
@@ -248,12 +257,15 @@ class BackwardMetadata:
 
 
 def compute_backward_metadata(mask: torch.Tensor, pack_partial: bool = True) -> BackwardMetadata:
-    """``mask``: bool [B,H,Sq,Sk] (broadcast views are fine), Sq and Sk multiples of 128.
+    """``mask``: bool [B,H,Sq,Sk] (broadcast views are fine).  Sq and Sk that are not multiples of 128 are taken up to
+    the next one with rows and columns that attend to nothing, as :func:`sparse_attention_backward` does with its
+    tensors.
 
     ``pack_partial``: bit-pack the PARTIAL tiles of both tilings (2 * Sq*Sk/8 bytes per distinct plane at most) and
     drop the transposed copy; otherwise keep that copy (Sq*Sk bytes per distinct plane) for the key passes."""
     if mask.dim() != 4:
         raise ValueError("mask must be [B,H,Sq,Sk] (broadcast views are fine)")
+    mask = _pad_mask(mask, 128, 128)
     # the transposed mask as a tensor of its own, distinct planes only, so that its classification reads rows
     B, H = mask.shape[:2]
     distinct = mask[: 1 if mask.stride(0) == 0 else B, : 1 if mask.stride(1) == 0 else H]
@@ -281,7 +293,8 @@ def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor
 
     The reference has no backward pass (README.md:65 lists it as future work); this differentiates its forward
     (sparse_attn_kernel.py:149-185).  ``o`` and ``lse`` come from ``sparse_attention(..., return_lse=True)`` with the
-    same inputs.  D = 64 or 128, bf16/fp16, Sq and Sk multiples of 128.  The backward tiles the mask its own way
+    same inputs.  bf16/fp16; the kernels have D = 64 and 128 and tile by 128 rows, other head dims up to 128 and
+    other Sq, Sk are padded here (zero columns; rows that attend to nothing).  The backward tiles the mask its own way
     (128 x 64 both ways), whatever BLOCK_Q / BLOCK_K the forward used.  ``mask`` may be None when ``bwd_metadata``
     carries the packed PARTIAL tiles of both tilings.
     """
@@ -298,6 +311,15 @@ def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor
         assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
         if mask.device != q.device:
             raise ValueError("mask must be on the same device as q")
+    if Sq % 128 or Sk % 128:
+        # the kernels tile by 128 rows both ways: zero rows (lse = -inf: rows that attended to nothing) and mask rows
+        # and columns that attend to nothing are added, and the gradients of the added rows dropped
+        rows = lambda t, n: torch.nn.functional.pad(t, (0, 0, 0, -n % 128))  # noqa: E731
+        dq, dk, dv = sparse_attention_backward(
+            rows(do, Sq), rows(q, Sq), rows(k, Sk), rows(v, Sk), rows(o, Sq),
+            torch.nn.functional.pad(lse, (0, -Sq % 128), value=float("-inf")),
+            None if mask is None else _pad_mask(mask, 128, 128), bwd_metadata)
+        return dq[:, :, :Sq].contiguous(), dk[:, :, :Sk].contiguous(), dv[:, :, :Sk].contiguous()
     if bwd_metadata is None:
         if mask is None:
             raise ValueError("sparse_attention_backward needs the mask or a BackwardMetadata with packed tiles")

@@ -65,3 +65,23 @@ def test_backward(gpu, D):
     sparse_attention_trainable(qa, ka, va, me, 128, 32).backward(do)
     for g_, a in zip(got, (qa.grad, ka.grad, va.grad)):
         assert torch.equal(g_, a)
+
+
+@pytest.mark.parametrize("Sq,Sk,D", [(192, 320, 128), (96, 96, 64), (48, 208, 32)])
+def test_backward_sizes_not_multiples_of_128(gpu, Sq, Sk, D):
+    """The backward tiles by 128 rows both ways; other sizes are padded with rows that attend to nothing."""
+    B, H = 2, 2
+    q, k, v = W.qkv(B, H, Sq, D, torch.bfloat16, seed=Sq, device=gpu, Sk=Sk)
+    do = torch.randn(B, H, Sq, D, generator=torch.Generator().manual_seed(6)).to(gpu, torch.bfloat16)
+    mask = some_mask(Sq, Sk, gpu, Sk)
+    me = mask[None, None].expand(B, H, Sq, Sk)
+    q32, k32, v32 = (t.float().clone().requires_grad_(True) for t in (q, k, v))
+    F.scaled_dot_product_attention(q32, k32, v32, attn_mask=mask).backward(do.float())
+    want = (q32.grad, k32.grad, v32.grad)
+    BK = 16
+    for bmd in (None, compute_backward_metadata(me), compute_backward_metadata(me, pack_partial=False)):
+        qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+        sparse_attention_trainable(qa, ka, va, me, 16, BK, bwd_metadata=bmd).backward(do)
+        for g_, w, name in zip((qa.grad, ka.grad, va.grad), want, ("dq", "dk", "dv")):
+            assert g_.shape == w.shape
+            assert float((g_.float() - w).abs().max()) / max(1.0, float(w.abs().max())) <= TOL, name
