@@ -49,11 +49,13 @@ def kernel_tiles(Sq: int, Sk: int, D: int, BLOCK_Q: int, BLOCK_K: int):
     compiler accepts (sparse_attn_kernel.py:149-185); the result does not depend on them."""
     BLOCK_Q, BLOCK_K = int(BLOCK_Q), int(BLOCK_K)
     ok_k = BLOCK_K >= 16 and BLOCK_K & (BLOCK_K - 1) == 0 and Sk % BLOCK_K == 0
-    if Sq < 32:  # the few-rows kernels: one Q tile of all rows, KV tiles of 32 keys or more
+    if Sq < 32:  # the few-rows kernels: one Q tile of all rows, KV tiles of 32 keys or more, head dims up to 128
+        if D > 128:
+            return None
         if ok_k and BLOCK_K >= 32:
             return Sq, BLOCK_K
         return next(((Sq, bk) for bk in (32, 64) if Sk % bk == 0), None)
-    ok_q = [b for b in _KERNEL_BLOCK_Q if Sq % b == 0 and (D != 256 or b in (64, 128))]
+    ok_q = [b for b in _KERNEL_BLOCK_Q if Sq % b == 0 and (D <= 128 or b in (64, 128))]  # (D above 128 runs as 256)
     if not ok_q:
         return None
     bq = BLOCK_Q if BLOCK_Q in ok_q else ok_q[0]
@@ -92,12 +94,15 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
         mask = mask.expand(B, H, Sq, Sk)
     BLOCK_Q, BLOCK_K = int(BLOCK_Q), int(BLOCK_K)
     tiles = kernel_tiles(Sq, Sk, D, BLOCK_Q, BLOCK_K)
-    if tiles is None and mask is not None and Sq > 32 and Sq % BLOCK_Q == 0 and Sk % BLOCK_K == 0:
-        # More than 32 query rows, not a multiple of 32 (48, 80, ...): zero rows are added to q and all-False rows to
-        # the mask, and their (zero) output rows dropped again.  Nothing is kept between calls on this path.
-        padded_tiles = kernel_tiles(Sq + -Sq % 32, Sk, D, BLOCK_Q, BLOCK_K)
+    row_multiple = 32 if D <= 128 else 64  # the smallest Q tile the kernels have
+    if tiles is None and mask is not None and Sq % row_multiple and Sq % BLOCK_Q == 0 and Sk % BLOCK_K == 0:
+        # A row count that no Q tile of the kernels divides (48, 80, ...; fewer than 32 rows at a head dim the few-rows
+        # kernels do not have): zero rows are added to q and all-False rows to the mask, and their (zero) output rows
+        # dropped again.  Nothing is kept between calls on this path.
+        pad = -Sq % row_multiple
+        padded_tiles = kernel_tiles(Sq + pad, Sk, D, BLOCK_Q, BLOCK_K)
         if padded_tiles is not None:
-            out = sparse_attention(torch.nn.functional.pad(q, (0, 0, 0, -Sq % 32)), k, v, _pad_mask(mask, 32, 1),
+            out = sparse_attention(torch.nn.functional.pad(q, (0, 0, 0, pad)), k, v, _pad_mask(mask, row_multiple, 1),
                                    *padded_tiles, return_lse=return_lse)
             return (out[0][:, :, :Sq].contiguous(), out[1][:, :, :Sq].contiguous()) if return_lse \
                 else out[:, :, :Sq].contiguous()

@@ -35,6 +35,17 @@ def test_forward(gpu, D, dtype):
     assert (lse - torch.logsumexp(s.masked_fill(~mask, float("-inf")), dim=-1)).abs().max() <= 2e-2
 
 
+@pytest.mark.parametrize("D,Sq,BQ", [(192, 256, 32), (256, 256, 256), (192, 8, 8), (256, 24, 8), (160, 48, 16)])
+def test_wide_heads_with_tiles_and_rows_they_have_no_kernel_for(gpu, D, Sq, BQ):
+    B, H, Sk = 1, 2, 256
+    q, k, v = W.qkv(B, H, Sq, D, torch.bfloat16, seed=D + Sq, device=gpu, Sk=Sk)
+    mask = some_mask(Sq, Sk, gpu, D)
+    o = sparse_attention(q, k, v, mask, BQ, 32)
+    assert o.shape == q.shape
+    want = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), attn_mask=mask)
+    assert (o.float() - want).abs().max() <= TOL
+
+
 @pytest.mark.parametrize("D,Sq", [(32, 1), (96, 16), (80, 32)])
 def test_few_rows(gpu, D, Sq):
     B, H, Sk = 2, 2, 2048
