@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define SA_ABI_VERSION 11
+#define SA_ABI_VERSION 12
 
 enum sa_status {
     SA_OK = 0,
@@ -105,6 +105,28 @@ int sa_mask_classify(const uint8_t *mask, const int64_t mask_strides[4], int B, 
                      const int64_t full_lens_strides[3], int32_t *part_ids, const int64_t part_ids_strides[4],
                      int32_t *part_lens, const int64_t part_lens_strides[3], void *workspace,
                      size_t workspace_bytes, void *stream);
+
+/*
+ * sa_mask_classify for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference: its launcher allocates its outputs with
+ * torch.empty on every call (mask_utils.py:91-94) and has no scratch.  Same arguments, checks, kernels and results as
+ * sa_mask_classify, without `workspace`: the class bytes go to a device array of SA_STATIC_CLASSIFY_MAX_TILES bytes
+ * that belongs to the library (one copy per GPU it runs on, held until the process ends).  The call allocates and
+ * frees nothing.  The first call on a device asks the runtime for that array's address (hipGetSymbolAddress) and keeps
+ * it; make that first call outside a stream capture.
+ *
+ *   - More tiles over the distinct mask planes (sa_mask_classify_workspace_bytes) than SA_STATIC_CLASSIFY_MAX_TILES:
+ *     SA_ERR_WORKSPACE, nothing is launched.
+ *   - Every call on a GPU uses that GPU's one array: calls that may run at the same time on one GPU (two streams, two
+ *     threads) race on it; order them on one stream or with events.  Nothing needs clearing between calls: every byte
+ *     the second kernel reads is written by the first.
+ */
+#define SA_STATIC_CLASSIFY_MAX_TILES (1u << 20)
+int sa_mask_classify_static(const uint8_t *mask, const int64_t mask_strides[4], int B, int H, int Sq, int Sk, int BQ,
+                            int BK, int32_t *full_ids, const int64_t full_ids_strides[4], int32_t *full_lens,
+                            const int64_t full_lens_strides[3], int32_t *part_ids,
+                            const int64_t part_ids_strides[4], int32_t *part_lens,
+                            const int64_t part_lens_strides[3], void *stream);
 
 /*
  * Block-sparse flash-attention forward.  Replaces sparse_attention_kernel's launch

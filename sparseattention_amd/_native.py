@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsparseattn_hip.so")
 
-SA_ABI_VERSION = 11
+SA_ABI_VERSION = 12
 SA_OK = 0
 SA_ERR_INVALID_ARGUMENT = -1
 SA_ERR_UNSUPPORTED = -2
@@ -29,6 +29,7 @@ EXPORTS = (
     "sa_last_error",
     "sa_mask_classify_workspace_bytes",
     "sa_mask_classify",
+    "sa_mask_classify_static",
     "sa_sparse_attention_fwd",
     "sa_mask_pack_partial_bytes",
     "sa_mask_pack_partial",
@@ -81,6 +82,8 @@ def load() -> ctypes.CDLL:
     lib.sa_mask_classify.argtypes = (
         [_vp, _i64p] + [ctypes.c_int] * 6 + [_vp, _i64p] * 4 + [_vp, ctypes.c_size_t, _vp]
     )
+    lib.sa_mask_classify_static.restype = ctypes.c_int
+    lib.sa_mask_classify_static.argtypes = [_vp, _i64p] + [ctypes.c_int] * 6 + [_vp, _i64p] * 4 + [_vp]
     lib.sa_sparse_attention_fwd.restype = ctypes.c_int
     lib.sa_sparse_attention_fwd.argtypes = (
         [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [ctypes.c_int] * 8 + [ctypes.c_float, _vp]

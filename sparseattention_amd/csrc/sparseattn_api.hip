@@ -37,6 +37,109 @@ int check_tiling(int B, int H, int Sq, int Sk, int BQ, int BK) {
     return SA_OK;
 }
 
+// The two launches of the classification (class bytes, then compaction into the lists), after the argument checks
+// the entry points share.  `workspace` holds one class byte per tile of every distinct plane; the caller has checked
+// its size.  `who` names the entry point in error messages.
+int classify_impl(const char *who, const uint8_t *mask, const int64_t mask_strides[4], int B, int H, int Sq, int Sk,
+                  int BQ, int BK, int32_t *full_ids, const int64_t full_ids_strides[4], int32_t *full_lens,
+                  const int64_t full_lens_strides[3], int32_t *part_ids, const int64_t part_ids_strides[4],
+                  int32_t *part_lens, const int64_t part_lens_strides[3], void *workspace, void *stream) {
+    const int nQ = Sq / BQ, nK = Sk / BK;
+    const bool bcast_b = mask_strides[0] == 0 || B == 1;
+    const bool bcast_h = mask_strides[1] == 0 || H == 1;
+    // An output dimension may be folded (stride 0) only where every plane holds the same result.
+    const int64_t ob[4] = {full_ids_strides[0], full_lens_strides[0], part_ids_strides[0], part_lens_strides[0]};
+    const int64_t oh[4] = {full_ids_strides[1], full_lens_strides[1], part_ids_strides[1], part_lens_strides[1]};
+    int zb = 0, zh = 0;
+    for (int i = 0; i < 4; i++) {
+        zb += ob[i] == 0;
+        zh += oh[i] == 0;
+    }
+    if (B > 1 && zb != 0 && (zb != 4 || !bcast_b))
+        return fail(SA_ERR_INVALID_ARGUMENT, "%s: output batch stride 0 needs a batch-broadcast mask and must be 0 on all four outputs", who);
+    if (H > 1 && zh != 0 && (zh != 4 || !bcast_h))
+        return fail(SA_ERR_INVALID_ARGUMENT, "%s: output head stride 0 needs a head-broadcast mask and must be 0 on all four outputs", who);
+
+    sa::ClassifyParams cp{};
+    cp.mask = mask;
+    cp.sb = mask_strides[0];
+    cp.sh = mask_strides[1];
+    cp.sq = mask_strides[2];
+    cp.sk = mask_strides[3];
+    cp.cls = static_cast<uint8_t *>(workspace);
+    cp.uB = bcast_b ? 1 : B;
+    cp.uH = bcast_h ? 1 : H;
+    cp.Sq = Sq;
+    cp.Sk = Sk;
+    cp.BQ = BQ;
+    cp.BK = BK;
+    cp.nQ = nQ;
+    cp.nK = nK;
+    cp.lbk = log2_exact(BK);
+    if (nQ > 65535 || (int64_t)cp.uB * cp.uH > 65535)
+        return fail(SA_ERR_UNSUPPORTED, "%s: more than 65535 Q tiles or distinct mask planes", who);
+
+    // Wide kernel: 16-byte loads along a contiguous, aligned key dimension; a tile spans 1..64 lanes.
+    const bool wide = cp.lbk >= 4 && BK <= 1024 && (cp.sk == 1 || Sk == 1) && aligned(mask, 16) && cp.sq % 16 == 0 &&
+                      (cp.uB == 1 || cp.sb % 16 == 0) && (cp.uH == 1 || cp.sh % 16 == 0);
+    hipError_t e = sa::launch_classify(cp, wide, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "%s: classify launch failed: %s", who, hipGetErrorString(e));
+
+    sa::CompactParams kp{};
+    kp.cls = cp.cls;
+    kp.uH = cp.uH;
+    kp.bcast_b = bcast_b;
+    kp.bcast_h = bcast_h;
+    kp.oB = (B > 1 && zb == 4) ? 1 : B;
+    kp.oH = (H > 1 && zh == 4) ? 1 : H;
+    kp.nQ = nQ;
+    kp.nK = nK;
+    kp.full_ids = full_ids;
+    kp.full_lens = full_lens;
+    kp.part_ids = part_ids;
+    kp.part_lens = part_lens;
+    for (int i = 0; i < 4; i++) {
+        kp.fis[i] = full_ids_strides[i];
+        kp.pis[i] = part_ids_strides[i];
+    }
+    for (int i = 0; i < 3; i++) {
+        kp.fls[i] = full_lens_strides[i];
+        kp.pls[i] = part_lens_strides[i];
+    }
+    e = sa::launch_compact(kp, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "%s: compaction launch failed: %s", who, hipGetErrorString(e));
+    return SA_OK;
+}
+
+// Class bytes of sa_mask_classify_static: device memory that belongs to the library, one copy per GPU the library
+// runs on, held until the process ends.  Host code never uses this name as an address (on the host it is only a
+// stand-in for the symbol): static_scratch() asks the runtime for the array's address on the current device.
+constexpr size_t kStaticScratchBytes = SA_STATIC_CLASSIFY_MAX_TILES;
+static __device__ __align__(256) uint8_t scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices] = {};  // address of `scratch` on device i, once it has been asked for
+
+// Address of `scratch` on the current device (each GPU holds its own copy at its own address), or an error code
+// with the message set when the runtime does not give it.  The first call on a device asks the runtime, later calls
+// read the pointer kept then.  Two threads racing through the first call store the same value twice.
+int static_scratch(void **out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_mask_classify_static: hipGetDevice failed: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices)
+        return fail(SA_ERR_UNSUPPORTED, "sa_mask_classify_static: device ordinal %d (supported: below %d)", dev, kMaxDevices);
+    void *ptr = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (!ptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            return fail(SA_ERR_HIP, "sa_mask_classify_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+        __atomic_store_n(&g_scratch_ptr[dev], ptr, __ATOMIC_RELEASE);
+    }
+    *out = ptr;
+    return SA_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -66,72 +169,34 @@ int sa_mask_classify(const uint8_t *mask, const int64_t mask_strides[4], int B, 
     if (!workspace || workspace_bytes < need)
         return fail(SA_ERR_WORKSPACE, "sa_mask_classify: workspace of %zu bytes required, %zu given", need,
                     workspace ? workspace_bytes : (size_t)0);
+    return classify_impl("sa_mask_classify", mask, mask_strides, B, H, Sq, Sk, BQ, BK, full_ids, full_ids_strides,
+                         full_lens, full_lens_strides, part_ids, part_ids_strides, part_lens, part_lens_strides,
+                         workspace, stream);
+}
 
-    const int nQ = Sq / BQ, nK = Sk / BK;
-    const bool bcast_b = mask_strides[0] == 0 || B == 1;
-    const bool bcast_h = mask_strides[1] == 0 || H == 1;
-    // An output dimension may be folded (stride 0) only where every plane holds the same result.
-    const int64_t ob[4] = {full_ids_strides[0], full_lens_strides[0], part_ids_strides[0], part_lens_strides[0]};
-    const int64_t oh[4] = {full_ids_strides[1], full_lens_strides[1], part_ids_strides[1], part_lens_strides[1]};
-    int zb = 0, zh = 0;
-    for (int i = 0; i < 4; i++) {
-        zb += ob[i] == 0;
-        zh += oh[i] == 0;
-    }
-    if (B > 1 && zb != 0 && (zb != 4 || !bcast_b))
-        return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_classify: output batch stride 0 needs a batch-broadcast mask and must be 0 on all four outputs");
-    if (H > 1 && zh != 0 && (zh != 4 || !bcast_h))
-        return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_classify: output head stride 0 needs a head-broadcast mask and must be 0 on all four outputs");
-
-    sa::ClassifyParams cp{};
-    cp.mask = mask;
-    cp.sb = mask_strides[0];
-    cp.sh = mask_strides[1];
-    cp.sq = mask_strides[2];
-    cp.sk = mask_strides[3];
-    cp.cls = static_cast<uint8_t *>(workspace);
-    cp.uB = bcast_b ? 1 : B;
-    cp.uH = bcast_h ? 1 : H;
-    cp.Sq = Sq;
-    cp.Sk = Sk;
-    cp.BQ = BQ;
-    cp.BK = BK;
-    cp.nQ = nQ;
-    cp.nK = nK;
-    cp.lbk = log2_exact(BK);
-    if (nQ > 65535 || (int64_t)cp.uB * cp.uH > 65535)
-        return fail(SA_ERR_UNSUPPORTED, "sa_mask_classify: more than 65535 Q tiles or distinct mask planes");
-
-    // Wide kernel: 16-byte loads along a contiguous, aligned key dimension; a tile spans 1..64 lanes.
-    const bool wide = cp.lbk >= 4 && BK <= 1024 && (cp.sk == 1 || Sk == 1) && aligned(mask, 16) && cp.sq % 16 == 0 &&
-                      (cp.uB == 1 || cp.sb % 16 == 0) && (cp.uH == 1 || cp.sh % 16 == 0);
-    hipError_t e = sa::launch_classify(cp, wide, static_cast<hipStream_t>(stream));
-    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_mask_classify: classify launch failed: %s", hipGetErrorString(e));
-
-    sa::CompactParams kp{};
-    kp.cls = cp.cls;
-    kp.uH = cp.uH;
-    kp.bcast_b = bcast_b;
-    kp.bcast_h = bcast_h;
-    kp.oB = (B > 1 && zb == 4) ? 1 : B;
-    kp.oH = (H > 1 && zh == 4) ? 1 : H;
-    kp.nQ = nQ;
-    kp.nK = nK;
-    kp.full_ids = full_ids;
-    kp.full_lens = full_lens;
-    kp.part_ids = part_ids;
-    kp.part_lens = part_lens;
-    for (int i = 0; i < 4; i++) {
-        kp.fis[i] = full_ids_strides[i];
-        kp.pis[i] = part_ids_strides[i];
-    }
-    for (int i = 0; i < 3; i++) {
-        kp.fls[i] = full_lens_strides[i];
-        kp.pls[i] = part_lens_strides[i];
-    }
-    e = sa::launch_compact(kp, static_cast<hipStream_t>(stream));
-    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_mask_classify: compaction launch failed: %s", hipGetErrorString(e));
-    return SA_OK;
+int sa_mask_classify_static(const uint8_t *mask, const int64_t mask_strides[4], int B, int H, int Sq, int Sk, int BQ,
+                            int BK, int32_t *full_ids, const int64_t full_ids_strides[4], int32_t *full_lens,
+                            const int64_t full_lens_strides[3], int32_t *part_ids,
+                            const int64_t part_ids_strides[4], int32_t *part_lens,
+                            const int64_t part_lens_strides[3], void *stream) {
+    g_error[0] = 0;
+    if (!mask || !mask_strides || !full_ids || !full_ids_strides || !full_lens || !full_lens_strides || !part_ids ||
+        !part_ids_strides || !part_lens || !part_lens_strides)
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_mask_classify_static: null pointer argument");
+    if (const int rc = check_tiling(B, H, Sq, Sk, BQ, BK)) return rc;
+    const size_t need = sa_mask_classify_workspace_bytes(mask_strides, B, H, Sq, Sk, BQ, BK);
+    if (need > kStaticScratchBytes)
+        return fail(SA_ERR_WORKSPACE,
+                    "sa_mask_classify_static: %zu tiles over the distinct mask planes, the library's own scratch holds "
+                    "%zu (SA_STATIC_CLASSIFY_MAX_TILES); use sa_mask_classify with a workspace of the caller's",
+                    need, kStaticScratchBytes);
+    // Every class byte the compaction reads is written by the classification launch in front of it, so nothing of
+    // the previous call's contents has to be cleared.
+    void *ws = nullptr;
+    if (const int rc = static_scratch(&ws)) return rc;
+    return classify_impl("sa_mask_classify_static", mask, mask_strides, B, H, Sq, Sk, BQ, BK, full_ids,
+                         full_ids_strides, full_lens, full_lens_strides, part_ids, part_ids_strides, part_lens,
+                         part_lens_strides, ws, stream);
 }
 
 }  // extern "C"
