@@ -95,6 +95,10 @@ constexpr float kNegInf = -__builtin_inff();
 // Issued through inline assembly on purpose: the compiler then does not track it, so it does not hold
 // back later LDS reads of the OTHER buffer until the transfer lands.  Whoever reads the destination
 // must execute "s_waitcnt vmcnt(0)" and a workgroup barrier first (the main loop does).
+// The load takes its LDS address from m0, which needs a wait state after a scalar write.  The write of m0 and the
+// s_nop therefore stay INSIDE this asm statement: handing the address over as an "{m0}" input leaves the copy into
+// the (reserved) register to the compiler, with no guarantee of the wait state or that two loads do not share one
+// copy, and a build of that form ended in a GPU memory fault.
 __device__ __forceinline__ void dma16(const void *base, uint32_t lane_offset, uint32_t lds_addr) {
     // the base is wave-uniform by construction; say so in a way the register allocator cannot miss
     const uint64_t b = (uint64_t)(uintptr_t)base;

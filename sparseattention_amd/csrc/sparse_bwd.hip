@@ -75,8 +75,11 @@ __global__ __launch_bounds__(256, 2) void sparse_bwd_kernel(const BwdParams p) {
     const uint16_t *zbase = p.z + b * p.zs[0] + h * p.zs[1];
     const int32_t *fid = p.full_ids + b * p.fis[0] + h * p.fis[1] + rt * p.fis[2];
     const int32_t *pid = p.part_ids + b * p.pis[0] + h * p.pis[1] + rt * p.pis[2];
-    const int F = p.full_lens[b * p.fls[0] + h * p.fls[1] + rt * p.fls[2]];
-    const int T = F + p.part_lens[b * p.pls[0] + h * p.pls[1] + rt * p.pls[2]];  // chunks = list entries
+    // Counts and tile indices are clamped to the nS streamed tiles there are (the reference guards every K/V and mask
+    // load with kv_offset < SEQLEN_K, sparse_attn_kernel.py:35,39,60): stale or foreign metadata then gives wrong
+    // numbers, never an access outside the tensors or past the list's LDS copy (nS <= kBwdListCap, checked by the host).
+    const int F = min(max(p.full_lens[b * p.fls[0] + h * p.fls[1] + rt * p.fls[2]], 0), p.nS);
+    const int T = F + min(max(p.part_lens[b * p.pls[0] + h * p.pls[1] + rt * p.pls[2]], 0), p.nS - F);  // chunks = list entries
     const uint8_t *mrow = p.mask + b * p.ms[0] + h * p.ms[1] + (int64_t)rrow * p.mrs;
     // this lane's row in a packed tile: 8 bytes per row, 1024 per tile, nS tiles per resident tile
     const uint8_t *prow = p.packed + b * p.pks[0] + h * p.pks[1] + (int64_t)rt * p.nS * 1024 + (wave * 32 + l32) * 8;
@@ -148,7 +151,7 @@ __global__ __launch_bounds__(256, 2) void sparse_bwd_kernel(const BwdParams p) {
     // the tile's list (FULL entries, then PARTIAL ones) as first streamed rows
     for (int e = tid; e < T; e += 256) {
         const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
-        ent[e] = idx << 6;
+        ent[e] = min(max(idx, 0), p.nS - 1) << 6;
     }
     __syncthreads();
 

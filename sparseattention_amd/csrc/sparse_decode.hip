@@ -70,8 +70,12 @@ __global__ __launch_bounds__(kDecodeWaves * 64, 2) void sparse_decode_kernel(con
     const uint16_t *vbase = p.v + b * p.vs[0] + h * p.vs[1];
     const int32_t *fid = p.full_ids + b * p.fis[0] + h * p.fis[1];
     const int32_t *pid = p.part_ids + b * p.pis[0] + h * p.pis[1];
-    const int F = p.full_lens[b * p.fls[0] + h * p.fls[1]];
-    const int NE = F + p.part_lens[b * p.pls[0] + h * p.pls[1]];
+    // Counts and tile indices are clamped to what Sk holds (the reference guards every K/V and mask load with
+    // kv_offset < SEQLEN_K, sparse_attn_kernel.py:35,39,60): stale or foreign metadata then gives wrong numbers, never
+    // an access outside K, V or the mask.
+    const int nKt = p.Sk >> p.lbk;
+    const int F = min(max(p.full_lens[b * p.fls[0] + h * p.fls[1]], 0), nKt);
+    const int NE = F + min(max(p.part_lens[b * p.pls[0] + h * p.pls[1]], 0), nKt - F);
     const int sh = p.lbk - 5;  // chunks per list entry, log2
     const int T = NE << sh;
     // this workgroup's chunks [t_lo, t_hi); this wave takes t_lo + wave, + 4, ...
@@ -134,7 +138,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64, 2) void sparse_decode_kernel(con
     // list entry of chunk t -> first key column, PARTIAL or not
     auto idx_load = [&](int t) -> int {
         const int e = t >> sh;
-        return e < F ? fid[(int64_t)e * p.fis[2]] : pid[(int64_t)(e - F) * p.pis[2]];
+        const int idx = e < F ? fid[(int64_t)e * p.fis[2]] : pid[(int64_t)(e - F) * p.pis[2]];
+        return min(max(idx, 0), nKt - 1);
     };
     auto col_of = [&](int t, int idx) -> int {
         return (__builtin_amdgcn_readfirstlane(idx) << p.lbk) + ((t & ((1 << sh) - 1)) << 5);

@@ -125,12 +125,18 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
             return MODE == 2 ? (ne << (p.lbk - 6)) : ((ne + EPC - 1) / EPC);
         }
     };
+    // Counts are clamped to the nK tiles a row of tiles has, and an index outside [0, nK) becomes an ABSENT entry
+    // (tagged_entry, ps_list_deposit): the reference guards every K/V and mask load with kv_offset < SEQLEN_K
+    // (sparse_attn_kernel.py:35,39,60), so stale or foreign metadata must not become an access outside K, V, the
+    // packed tiles or the list's LDS copy.
+    auto clamp_full = [&](int F_) -> int { return min(max(F_, 0), p.nK); };
+    auto clamp_part = [&](int F_, int P_) -> int { return min(max(P_, 0), p.nK - clamp_full(F_)); };
     auto set_item = [&](int b_, int h_, int qt_, int F_, int P_) {
         b = b_;
         h = h_;
         qt = qt_;
-        F = F_;
-        NE = F_ + P_;
+        F = clamp_full(F_);
+        NE = F + clamp_part(F_, P_);
         T = chunks_of(NE);
         kbase = p.k + b * p.ks[0] + h * p.ks[1];
         vbase = p.v + b * p.vs[0] + h * p.vs[1];
@@ -257,6 +263,7 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
     auto tagged_entry = [&](int e) -> int {  // from global memory
         if (e >= NE) return kAbsent;
         const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
+        if ((unsigned)idx >= (unsigned)p.nK) return kAbsent;
         return (MODE == 2 ? (idx << p.lbk) : (idx << LBKC)) | (e >= F ? kPartialBit : 0);
     };
     if (list_in_lds) {
@@ -319,7 +326,9 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
 #pragma unroll
         for (int i = 0; i < PER; i++) {
             const int e = tid + NT * i;
-            if (e < cnt) dst[e] = e >= ne ? kAbsent : ((lr[i] << lbk_rt) | (e >= F_ ? kPartialBit : 0));
+            if (e < cnt)
+                dst[e] = (e >= ne || (unsigned)lr[i] >= (unsigned)p.nK) ? kAbsent
+                                                                         : ((lr[i] << lbk_rt) | (e >= F_ ? kPartialBit : 0));
         }
     };
     auto ps_entries_read = [&](const int *el, int t, int(&raw)[EPC]) {
@@ -702,13 +711,13 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
         ps_list_deposit(F, NE - F, lr, elist(0));
         if (has_nx) {
             const int4 e1 = sched_row[2];
-            nx_bh = rfl(e1.x), nx_qt = rfl(e1.y), nx_F = rfl(e1.z), nx_P = rfl(e1.w);
+            nx_bh = rfl(e1.x), nx_qt = rfl(e1.y), nx_F = clamp_full(rfl(e1.z)), nx_P = clamp_part(rfl(e1.z), rfl(e1.w));
             ps_list_issue(nx_bh >> 16, nx_bh & 0xffff, nx_qt, nx_F, nx_P, lr);
             ps_list_deposit(nx_F, nx_P, lr, elist(1));
         }
         if (has_n2) {
             const int4 e2 = sched_row[3];
-            n2_bh = rfl(e2.x), n2_qt = rfl(e2.y), n2_F = rfl(e2.z), n2_P = rfl(e2.w);
+            n2_bh = rfl(e2.x), n2_qt = rfl(e2.y), n2_F = clamp_full(rfl(e2.z)), n2_P = clamp_part(rfl(e2.z), rfl(e2.w));
             ps_list_issue(n2_bh >> 16, n2_bh & 0xffff, n2_qt, n2_F, n2_P, lr);  // stays in registers for now
         }
         int4 e3 = 3 < n_items ? sched_row[4] : int4{0, 0, 0, 0};
@@ -825,7 +834,7 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
                 nx_bh = n2_bh, nx_qt = n2_qt, nx_F = n2_F, nx_P = n2_P;
                 has_n2 = it + 2 < n_items;
                 if (has_n2) {
-                    n2_bh = rfl(e3.x), n2_qt = rfl(e3.y), n2_F = rfl(e3.z), n2_P = rfl(e3.w);
+                    n2_bh = rfl(e3.x), n2_qt = rfl(e3.y), n2_F = clamp_full(rfl(e3.z)), n2_P = clamp_part(rfl(e3.z), rfl(e3.w));
                     ps_list_issue(n2_bh >> 16, n2_bh & 0xffff, n2_qt, n2_F, n2_P, lr);
                 }
                 if (it + 3 < n_items) e3 = sched_row[1 + it + 3];

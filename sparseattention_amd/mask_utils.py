@@ -114,6 +114,10 @@ def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int, pack_par
                         schedule=None) -> MaskMetadata:
     """Classify the mask's tiles on the GPU (replaces mask_utils.py:85-107).
 
+    Memory beyond the reference's four tensors: with ``pack_partial`` (the default when BLOCK_K is a multiple of 8)
+    ``Sq*Sk/8`` bytes per DISTINCT mask plane for ``packed_masks`` (128 MiB for a [32768,32768] mask; B*H times that
+    for a mask that differs per batch element and head).  ``pack_partial=False`` allocates only the four tensors.
+
     ``mask``: bool [B,H,Sq,Sk] on a ROCm device, any strides.  Dimensions that are broadcast in
     ``mask`` (stride 0, e.g. from ``mask.expand(B,H,Sq,Sk)``) are classified once and the returned
     tensors are broadcast views over them, so every ``[b,h]`` plane reads the same values the
@@ -173,7 +177,9 @@ def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int, pack_par
             _native.check(rc)
             packed = packed.expand(B, H, nQ, nK, BLOCK_Q * BLOCK_K // 8)
         sched, mode = _make_schedule(lib, fl, pl, B, H, Sq, Sk, BLOCK_Q, BLOCK_K, schedule, dev)
-    return MaskMetadata(fid, fl, pid, pl, packed, sched, mode)
+    md = MaskMetadata(fid, fl, pid, pl, packed, sched, mode)
+    md._validated_for = (int(Sk), int(BLOCK_K))  # lists made by the kernels above fit these sizes by construction
+    return md
 
 
 # Tile sizes tried by select_block_sizes, and what one executed mask entry costs at each BLOCK_Q relative to
@@ -356,4 +362,6 @@ def compute_mask_terms(terms: Sequence[MaskTerm], B: int, H: int, Sq: int, Sk: i
         _native.check(rc)
         del workspace
         sched, mode = _make_schedule(lib, fl, pl, B, H, Sq, Sk, BLOCK_Q, BLOCK_K, schedule, dev)
-    return MaskMetadata(fid, fl, pid, pl, packed, sched, mode)
+    md = MaskMetadata(fid, fl, pid, pl, packed, sched, mode)
+    md._validated_for = (int(Sk), int(BLOCK_K))  # lists made by the kernels above fit these sizes by construction
+    return md

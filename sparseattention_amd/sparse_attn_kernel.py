@@ -39,6 +39,49 @@ def _pad_mask(mask: torch.Tensor, q_multiple: int, k_multiple: int) -> torch.Ten
     return padded.expand(B, H, *padded.shape[2:])
 
 
+def _same_device(ref: torch.Tensor, **tensors) -> None:
+    """Every tensor whose data pointer goes to a kernel must live where ``ref`` lives: a host pointer (or one of
+    another GPU) in any slot would be a memory fault on the device, where the reference raises a Python error."""
+    for name, t in tensors.items():
+        if t is not None and t.device != ref.device:
+            raise ValueError(f"{name} is on {t.device}, expected {ref.device} (every tensor argument must be on q's device)")
+
+
+def validate_metadata(md: MaskMetadata, Sk: int, BLOCK_K: int) -> None:
+    """Raise ValueError unless the lists can address K and V: ``0 <= lens``, ``unmasked_lens + masked_lens <= Sk/BLOCK_K``
+    and ``0 <= ids[..., :len] < Sk/BLOCK_K`` (the reference guards its loads with ``kv_offset < SEQLEN_K``,
+    sparse_attn_kernel.py:35,39,60).  Plain torch on the tensors' own device; reads two flags back, so it synchronises.
+    The wrappers run it once per metadata object that did not come from this package's own preprocessing; the kernels
+    additionally clamp counts and skip indices out of range, so unchecked metadata cannot fault either."""
+    nK = Sk // BLOCK_K
+    bad = []
+    fl, pl = md.unmasked_lens, md.masked_lens
+    if bool(((fl < 0) | (pl < 0) | (fl.to(torch.int64) + pl.to(torch.int64) > nK)).any()):
+        bad.append(f"counts outside [0, {nK}] or unmasked_lens + masked_lens > {nK}")
+    for name, ids, lens in (("unmasked_kv_ids", md.unmasked_kv_ids, fl), ("masked_kv_ids", md.masked_kv_ids, pl)):
+        if ids.shape[-1] != nK:
+            bad.append(f"{name} has {ids.shape[-1]} slots per Q tile, expected {nK}")
+            continue
+        live = torch.arange(nK, device=ids.device) < lens[..., None]
+        if bool((live & ((ids < 0) | (ids >= nK))).any()):
+            bad.append(f"{name}[..., :len] holds tile indices outside [0, {nK})")
+    if bad:
+        raise ValueError("mask_metadata does not fit Sk=%d, BLOCK_K=%d: %s" % (Sk, BLOCK_K, "; ".join(bad)))
+
+
+def _checked_metadata(md: MaskMetadata, Sk: int, BLOCK_K: int) -> None:
+    """validate_metadata once per (object, tiling); metadata made by compute_mask_kernel / compute_mask_terms is
+    trusted (marked there), so the usual call path never synchronises."""
+    key = (int(Sk), int(BLOCK_K))
+    if getattr(md, "_validated_for", None) == key:
+        return
+    validate_metadata(md, Sk, BLOCK_K)
+    try:
+        md._validated_for = key
+    except AttributeError:  # a carrier that takes no new attributes is simply checked again next time
+        pass
+
+
 _KERNEL_BLOCK_Q = (128, 64, 32, 256)  # in order of preference when the caller's size is not one of them
 
 
@@ -86,8 +129,10 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
         raise ValueError(f"k/v shapes {tuple(k.shape)}/{tuple(v.shape)} do not match q {tuple(q.shape)}")
     if not q.is_cuda:
         raise RuntimeError("sparse_attention needs q, k, v on a ROCm GPU; there is no CPU path")
+    _same_device(q, k=k, v=v, mask=mask)
     if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
-        raise TypeError(f"q, k, v must share dtype bfloat16 or float16 (got {q.dtype}, {k.dtype}, {v.dtype})")
+        raise TypeError(f"q, k, v must share dtype bfloat16 or float16 (got {q.dtype}, {k.dtype}, {v.dtype}); "
+                        "float32 inputs, which the reference's kernel accepts, have no kernel here: cast them")
     if mask is None and getattr(mask_metadata, "packed_masks", None) is None:
         raise ValueError("sparse_attention without a mask tensor needs mask_metadata with packed_masks")
     if mask is not None:
@@ -124,9 +169,11 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
         BLOCK_Q, BLOCK_K = tiles
         mask_metadata = again[1]
 
-    if (Sq == BLOCK_Q and Sq < 32 and BLOCK_K >= 32 and getattr(mask_metadata, "packed_masks", None) is None
-            and getattr(mask_metadata, "schedule", None) is None):
-        # one Q tile of fewer rows than the forward kernels tile by: the split-KV kernels
+    if Sq == BLOCK_Q and Sq < 32 and BLOCK_K >= 32:
+        # one Q tile of fewer rows than the forward kernels tile by: the split-KV kernels.  They read the bool mask and
+        # use neither packed tiles nor a schedule, so metadata that carries those (compute_mask_kernel's default) runs too.
+        if mask is None:
+            raise ValueError("sparse_attention with fewer than 32 query rows reads the mask tensor: pass `mask`")
         return sparse_attention_decode(q, k, v, mask, BLOCK_K, mask_metadata, return_lse=return_lse)
     sm_scale = D ** (-0.5) * 1 / math.log(2)  # exp2 replaces exp (sparse_attn_kernel.py:152)
 
@@ -139,10 +186,9 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
                            ("unmasked_lens", fl, (B, H, nQ)), ("masked_lens", pl, (B, H, nQ))):
         if tuple(t.shape) != shape or t.dtype != torch.int32 or t.device != q.device:
             raise ValueError(f"mask_metadata.{name}: expected int32 {shape} on {q.device}, got {t.dtype} {tuple(t.shape)} on {t.device}")
+    _checked_metadata(mask_metadata, Sk, BLOCK_K)
     if mask is not None:
         assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
-        if mask.device != q.device:
-            raise ValueError("mask must be on the same device as q")
     packed = getattr(mask_metadata, "packed_masks", None)
     if packed is not None:
         shape = (B, H, nQ, nK, BLOCK_Q * BLOCK_K // 8)
@@ -205,6 +251,7 @@ def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, m
         raise ValueError(f"k/v shapes {tuple(k.shape)}/{tuple(v.shape)} do not match q {tuple(q.shape)}")
     if not q.is_cuda:
         raise RuntimeError("sparse_attention_decode needs q, k, v on a ROCm GPU; there is no CPU path")
+    _same_device(q, k=k, v=v, mask=mask)
     if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
         raise TypeError(f"q, k, v must share dtype bfloat16 or float16 (got {q.dtype}, {k.dtype}, {v.dtype})")
     sm_scale = D ** (-0.5) * 1 / math.log(2)
@@ -218,9 +265,8 @@ def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, m
                            ("unmasked_lens", fl, (B, H, 1)), ("masked_lens", pl, (B, H, 1))):
         if tuple(t.shape) != shape or t.dtype != torch.int32 or t.device != q.device:
             raise ValueError(f"mask_metadata.{name}: expected int32 {shape} on {q.device}, got {t.dtype} {tuple(t.shape)} on {t.device}")
+    _checked_metadata(mask_metadata, Sk, BLOCK_K)
     assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
-    if mask.device != q.device:
-        raise ValueError("mask must be on the same device as q")
     Dk = _kernel_head_dim(D, (64, 128))
     qc, kc, vc = (_kernel_ready(_pad_head_dim(t, Dk)) for t in (q, k, v))
     o = torch.empty_like(qc)
@@ -307,15 +353,17 @@ def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor
     Sk = k.shape[-2]
     if not q.is_cuda:
         raise RuntimeError("sparse_attention_backward needs its tensors on a ROCm GPU; there is no CPU path")
+    _same_device(q, k=k, v=v, o=o, do=do, lse=lse, mask=mask)
     if q.dtype not in _DTYPES or any(t.dtype != q.dtype for t in (k, v, o, do)):
         raise TypeError("q, k, v, o, do must share dtype bfloat16 or float16")
+    if k.shape != (B, H, Sk, D) or v.shape != k.shape or o.shape != q.shape or do.shape != q.shape:
+        raise ValueError(f"shapes: q/o/do must be {(B, H, Sq, D)} and k/v {(B, H, Sk, D)} (got q {tuple(q.shape)}, "
+                         f"k {tuple(k.shape)}, v {tuple(v.shape)}, o {tuple(o.shape)}, do {tuple(do.shape)})")
     if lse.dtype != torch.float32 or tuple(lse.shape) != (B, H, Sq):
         raise ValueError(f"lse: expected float32 {(B, H, Sq)}, got {lse.dtype} {tuple(lse.shape)}")
     if mask is not None:
         mask = mask.expand(B, H, Sq, Sk)
         assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
-        if mask.device != q.device:
-            raise ValueError("mask must be on the same device as q")
     if Sq % 128 or Sk % 128:
         # the kernels tile by 128 rows both ways: zero rows (lse = -inf: rows that attended to nothing) and mask rows
         # and columns that attend to nothing are added, and the gradients of the added rows dropped
@@ -342,6 +390,7 @@ def sparse_attention_backward(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor
             if tuple(t.shape) != shp or t.dtype != torch.int32 or t.device != q.device:
                 raise ValueError(f"bwd_metadata: expected int32 {shp} on {q.device}, got {t.dtype} {tuple(t.shape)}")
             lists += [t.data_ptr(), S(t.stride())]
+        _checked_metadata(md, 64 * shape[3], 64)
         pk = getattr(md, "packed_masks", None)
         if pk is not None and (tuple(pk.shape) != shape + (1024,) or pk.dtype != torch.uint8 or pk.device != q.device
                                or pk.stride()[2:] != (shape[3] * 1024, 1024, 1)):
@@ -403,6 +452,7 @@ def merge_attention_parts(o_parts: torch.Tensor, lse_parts: torch.Tensor, return
         raise ValueError("o_parts must be [n,B,H,Sq,D] and lse_parts float32 [n,B,H,Sq]")
     if o_parts.dtype not in _DTYPES or not o_parts.is_cuda:
         raise TypeError("o_parts must be a bfloat16 or float16 tensor on a ROCm GPU")
+    _same_device(o_parts, lse_parts=lse_parts)
     n, B, H, Sq, D = o_parts.shape
     if o_parts.stride(-1) != 1 or o_parts.data_ptr() % 16 or any(s % 8 for s in o_parts.stride()[:-1]):
         o_parts = o_parts.contiguous()

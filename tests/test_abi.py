@@ -198,3 +198,55 @@ def test_product_code_never_touches_the_oracle():
                 text = open(os.path.join(dirpath, f)).read()
                 assert not re.search(r"^\s*(import|from)\s+oracle\b", text, flags=re.M), f
                 assert "liboracle" not in text, f
+
+
+def test_reference_import_paths_give_the_same_objects():
+    # the reference's callers: from sparseattention.sparse_attn_kernel import sparse_attention;
+    # from sparseattention.mask_utils import compute_mask_kernel (test_attn.py:11-12)
+    import sparseattention.mask_utils as ref_mu
+    import sparseattention.sparse_attn_kernel as ref_sa
+    import sparseattention.test_attn as ref_ta
+    import sparseattention_amd
+    from sparseattention.mask_utils import MaskMetadata, compute_mask_kernel, compute_mask_slow
+    from sparseattention.sparse_attn_kernel import sparse_attention
+
+    assert sparse_attention is sparseattention_amd.sparse_attention is ref_sa.sparse_attention
+    assert compute_mask_kernel is sparseattention_amd.compute_mask_kernel is ref_mu.compute_mask_kernel
+    assert compute_mask_slow is sparseattention_amd.compute_mask_slow
+    assert MaskMetadata is sparseattention_amd.MaskMetadata
+    assert ref_ta.random_blocked_mask is sparseattention_amd.test_attn.random_blocked_mask
+    import dataclasses
+    assert [f.name for f in dataclasses.fields(MaskMetadata)][:4] == ["unmasked_kv_ids", "unmasked_lens", "masked_kv_ids",
+                                                                     "masked_lens"]
+
+
+def test_validate_metadata_on_cpu_tensors():
+    from sparseattention_amd import compute_mask_slow
+    from sparseattention_amd.sparse_attn_kernel import validate_metadata
+
+    mask = (torch.rand(1, 2, 256, 256, generator=torch.Generator().manual_seed(0)) < 0.5)
+    mask[0, 0, :64, :64] = True
+    mask[0, 1, 64:128, 64:192] = False
+    md = compute_mask_slow(mask, 64, 32)
+    validate_metadata(md, 256, 32)  # the -1 in unused slots is fine
+    with pytest.raises(ValueError, match="slots per Q tile"):
+        validate_metadata(md, 512, 32)
+    md.unmasked_lens = md.unmasked_lens.clone()
+    md.unmasked_lens[0, 0, 0] += 1  # (the tile row holds PARTIAL tiles, so the next slot is a -1)
+    with pytest.raises(ValueError, match=r"unmasked_kv_ids\[\.\.\., :len\]"):
+        validate_metadata(md, 256, 32)
+    md.unmasked_lens[0, 0, 0] = -1
+    with pytest.raises(ValueError, match="counts"):
+        validate_metadata(md, 256, 32)
+    md.unmasked_lens[0, 0, 0] = 9
+    with pytest.raises(ValueError, match="counts"):
+        validate_metadata(md, 256, 32)
+
+
+def test_device_check_names_the_tensor():
+    from sparseattention_amd.sparse_attn_kernel import _same_device
+
+    ref = torch.empty(1, device="meta")
+    _same_device(ref, k=torch.empty(2, device="meta"), mask=None)
+    with pytest.raises(ValueError, match="lse is on cpu"):
+        _same_device(ref, k=torch.empty(2, device="meta"), lse=torch.empty(2))

@@ -1,0 +1,228 @@
+"""What the wrappers and kernels do with arguments the reference would reject or guard: tensors on the wrong device
+(the reference's launcher raises a Python error), tile lists that do not fit Sk (the reference masks every K/V and
+mask load with kv_offset < SEQLEN_K, sparse_attn_kernel.py:35,39,60), and the exact CPU-plumbing workload on the GPU."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from helpers import assert_metadata_equal
+from sparseattention_amd import (MaskMetadata, _native, compute_backward_metadata, compute_mask_kernel,
+                                 compute_mask_slow, sparse_attention, sparse_attention_backward,
+                                 sparse_attention_decode, workloads as W)
+from sparseattention_amd.sparse_attn_kernel import merge_attention_parts, validate_metadata
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+
+
+def sdpa32(q, k, v, mask):
+    return F.scaled_dot_product_attention(q.float(), k.float(), v.float(), attn_mask=mask)
+
+
+def test_tensors_on_the_wrong_device_raise_before_any_launch(gpu):
+    B, H, S, D = 1, 2, 256, 64
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=1, device=gpu)
+    mask = W.causal_mask(S, gpu)
+    md = compute_mask_kernel(mask[None, None].expand(B, H, S, S), 128, 32)
+    for bad in ("k", "v", "mask"):
+        args = {"k": k, "v": v, "mask": mask}
+        args[bad] = args[bad].cpu()
+        with pytest.raises(ValueError, match=bad):
+            sparse_attention(q, args["k"], args["v"], args["mask"], 128, 32, mask_metadata=md)
+    with pytest.raises(ValueError, match="v is on cpu"):
+        sparse_attention_decode(q[:, :, :8], k, v.cpu(), mask[:8], 32)
+    o, lse = sparse_attention(q, k, v, mask, 128, 32, return_lse=True)
+    do = torch.ones_like(o)
+    for bad in ("k", "o", "do", "lse"):
+        a = {"do": do, "k": k, "o": o, "lse": lse}
+        a[bad] = a[bad].cpu()
+        with pytest.raises(ValueError, match=f"{bad} is on cpu"):
+            sparse_attention_backward(a["do"], q, a["k"], v, a["o"], a["lse"], mask)
+    with pytest.raises(ValueError, match="lse_parts is on cpu"):
+        merge_attention_parts(o[None], lse[None].cpu())
+    # metadata on the host (e.g. from compute_mask_slow on a CPU mask)
+    with pytest.raises(ValueError, match="mask_metadata"):
+        sparse_attention(q, k, v, mask, 128, 32, mask_metadata=compute_mask_slow(mask.cpu()[None, None].expand(B, H, S, S), 128, 32))
+
+
+def test_metadata_that_does_not_fit_is_refused_by_the_wrappers(gpu):
+    B, H, S, D, BQ, BK = 1, 1, 512, 64, 128, 32
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=2, device=gpu)
+    mask = W.random_block_mask(S, 32, 0.5, seed=2, device=gpu)[None, None]
+    good = compute_mask_kernel(mask, BQ, BK, pack_partial=False)
+    # the lists of compute_mask_slow (unused slots hold -1) are fine
+    slow = compute_mask_slow(mask, BQ, BK)
+    assert torch.equal(sparse_attention(q, k, v, mask, BQ, BK, mask_metadata=slow),
+                       sparse_attention(q, k, v, mask, BQ, BK, mask_metadata=good))
+    clone = lambda md: MaskMetadata(md.unmasked_kv_ids.clone(), md.unmasked_lens.clone(), md.masked_kv_ids.clone(),  # noqa: E731
+                                    md.masked_lens.clone())
+    stale = clone(slow)
+    stale.unmasked_lens[0, 0, 1] += 1  # reaches into the -1 slots
+    with pytest.raises(ValueError, match="unmasked_kv_ids"):
+        sparse_attention(q, k, v, mask, BQ, BK, mask_metadata=stale)
+    long = clone(good)
+    long.masked_lens[0, 0, 0] = S // BK + 1
+    with pytest.raises(ValueError, match="counts"):
+        sparse_attention(q, k, v, mask, BQ, BK, mask_metadata=long)
+    # lists made for a longer Sk: indices past this Sk
+    other = compute_mask_kernel(torch.ones(1, 1, S, 2 * S, dtype=torch.bool, device=gpu), BQ, BK, pack_partial=False)
+    with pytest.raises(ValueError):
+        validate_metadata(other, S, BK)
+
+
+def _fwd_raw(q, k, v, mask, md, BQ, BK, packed=None):
+    """The forward straight through the C ABI (no validation of the lists on the way)."""
+    lib = _native.load()
+    S = _native.strides
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    o = torch.full_like(q, float("nan"))
+    me = mask.expand(B, H, Sq, Sk)
+    rc = lib.sa_sparse_attention_fwd_ex(
+        q.data_ptr(), S(q.stride()), k.data_ptr(), S(k.stride()), v.data_ptr(), S(v.stride()), o.data_ptr(), S(o.stride()),
+        me.data_ptr(), S(me.stride()),
+        md.unmasked_kv_ids.data_ptr(), S(md.unmasked_kv_ids.stride()), md.unmasked_lens.data_ptr(), S(md.unmasked_lens.stride()),
+        md.masked_kv_ids.data_ptr(), S(md.masked_kv_ids.stride()), md.masked_lens.data_ptr(), S(md.masked_lens.stride()),
+        packed.data_ptr() if packed is not None else None, S(packed.stride()[:2]) if packed is not None else None,
+        None, 0, 0, B, H, Sq, Sk, D, BQ, BK, 0, D ** -0.5 / math.log(2), torch.cuda.current_stream().cuda_stream)
+    _native.check(rc)
+    torch.cuda.synchronize()
+    return o
+
+
+@pytest.mark.parametrize("BK", [16, 32, 64])
+def test_kernels_skip_list_entries_that_do_not_fit(gpu, BK):
+    # Through the C ABI, lists with counts beyond the row of tiles and indices outside [0, Sk/BK): the forward treats
+    # such entries as absent, so the result is that of the mask without those tiles.
+    B, H, S, D, BQ = 1, 2, 512, 64, 128
+    nK = S // BK
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=3, device=gpu)
+    mask = W.random_block_mask(S, 64, 0.4, seed=3, device=gpu)
+    me = mask[None, None].expand(B, H, S, S)
+    md = compute_mask_kernel(me, BQ, BK, pack_partial=True)
+    bad = MaskMetadata(md.unmasked_kv_ids.contiguous().clone(), md.unmasked_lens.contiguous().clone(),
+                       md.masked_kv_ids.contiguous().clone(), md.masked_lens.contiguous().clone())
+    pos = torch.arange(nK, device=gpu)
+    for ids, lens in ((bad.unmasked_kv_ids, bad.unmasked_lens), (bad.masked_kv_ids, bad.masked_lens)):
+        ids[pos.expand_as(ids) >= lens[..., None]] = 1 << 28  # what torch.empty may leave in the unused slots
+    expect_mask = me.clone()
+    # one FULL and one PARTIAL entry of Q tile 1 (both planes) point outside: those tiles drop out
+    for ids, lens, repl in ((bad.unmasked_kv_ids, bad.unmasked_lens, nK + 3), (bad.masked_kv_ids, bad.masked_lens, -1)):
+        assert int(lens[0, 0, 1]) >= 1
+        tile = int(ids[0, 0, 1, 0])
+        ids[:, :, 1, 0] = repl
+        expect_mask[:, :, BQ:2 * BQ, tile * BK:(tile + 1) * BK] = False
+    # counts beyond the row: the slots they reach hold indices out of range, which are skipped.  A FULL count that
+    # takes the whole row of tiles leaves no room for PARTIAL entries: Q tile 2 keeps its FULL tiles only.
+    bad.unmasked_lens[:, :, 2] = nK + 100
+    expect_mask[:, :, 2 * BQ:3 * BQ] &= _tiles_mask(md.unmasked_kv_ids, md.unmasked_lens, 2, BQ, BK, S, gpu)
+    bad.masked_lens[:, :, 3] = 1 << 20
+    bad.unmasked_lens[:, :, 0] = -5  # a negative count reads as 0
+    expect_mask[:, :, :BQ] &= ~_tiles_mask(md.unmasked_kv_ids, md.unmasked_lens, 0, BQ, BK, S, gpu)
+    want = sdpa32(q, k, v, expect_mask)
+    dead = ~expect_mask.any(-1)
+    want[dead] = 0.0
+    for packed in (None, md.packed_masks):
+        o = _fwd_raw(q, k, v, mask, bad, BQ, BK, packed)
+        assert torch.isfinite(o).all()
+        assert (o.float() - want).abs().max() <= TOL
+
+
+def _tiles_mask(ids, lens, qt, BQ, BK, S, dev):
+    """bool [B,H,BQ,S]: the key columns of the listed tiles of Q tile qt."""
+    B, H = ids.shape[:2]
+    out = torch.zeros(B, H, 1, S, dtype=torch.bool, device=dev)
+    for b in range(B):
+        for h in range(H):
+            for j in ids[b, h, qt, :int(lens[b, h, qt])].tolist():
+                out[b, h, 0, j * BK:(j + 1) * BK] = True
+    return out.expand(B, H, BQ, S)
+
+
+def test_decode_and_backward_stay_inside_their_tensors_with_lists_that_do_not_fit(gpu):
+    # C ABI, counts beyond the row of tiles and indices out of range: the kernels clamp both (results are then those
+    # of other tiles, as with the reference's masked loads), every access stays inside K, V and the mask.
+    lib = _native.load()
+    S = _native.strides
+    B, H, Sq, Sk, D, BK = 1, 2, 8, 1024, 64, 32
+    q, k, v = W.qkv(B, H, Sq, D, torch.bfloat16, seed=4, device=gpu, Sk=Sk)
+    mask = (torch.rand(Sq, Sk, generator=torch.Generator().manual_seed(4)) < 0.5).to(gpu)
+    me = mask[None, None].expand(B, H, Sq, Sk)
+    md = compute_mask_kernel(me, Sq, BK, pack_partial=False)
+    fid, pid = md.unmasked_kv_ids.contiguous().clone(), md.masked_kv_ids.contiguous().clone()
+    fl, pl = md.unmasked_lens.contiguous().clone(), md.masked_lens.contiguous().clone()
+    fid[:] = 1 << 27
+    pid[..., 1::2] = -3
+    fl[:] = 7
+    pl[:] = Sk // BK + 9
+    o = torch.empty_like(q)
+    rc = lib.sa_sparse_attention_decode(
+        q.data_ptr(), S(q.stride()), k.data_ptr(), S(k.stride()), v.data_ptr(), S(v.stride()), o.data_ptr(), S(o.stride()),
+        me.data_ptr(), S(me.stride()), fid.data_ptr(), S(fid.stride()), fl.data_ptr(), S(fl.stride()),
+        pid.data_ptr(), S(pid.stride()), pl.data_ptr(), S(pl.stride()), B, H, Sq, Sk, D, BK, 0, D ** -0.5 / math.log(2),
+        1, None, 0, None, None, torch.cuda.current_stream().cuda_stream)
+    _native.check(rc)
+    torch.cuda.synchronize()
+    assert not torch.isnan(o).any()
+
+    # backward: valid lists first (the expected gradients), then the same call with corrupted copies
+    B, H, S, D = 1, 2, 256, 64
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=5, device=gpu)
+    mask = W.causal_mask(S, gpu)[None, None].expand(B, H, S, S)
+    o, lse = sparse_attention(q, k, v, mask, 128, 32, return_lse=True)
+    do = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(6)).to(gpu, torch.bfloat16)
+    bmd = compute_backward_metadata(mask, pack_partial=False)
+    good = sparse_attention_backward(do, q, k, v, o, lse, mask, bmd)
+    for md in (bmd.by_query, bmd.by_key):
+        for name in ("unmasked_kv_ids", "unmasked_lens", "masked_kv_ids", "masked_lens"):
+            setattr(md, name, getattr(md, name).contiguous().clone())
+        md.unmasked_kv_ids[..., 0] = 1 << 25
+        md.masked_kv_ids[..., 0] = -1
+        md.unmasked_lens[:] = 1 << 16
+        md.masked_lens[:] = -4
+        md._validated_for = (S, 64)  # straight to the kernels
+    got = sparse_attention_backward(do, q, k, v, o, lse, mask, bmd)
+    torch.cuda.synchronize()
+    assert all(g.shape == w.shape for g, w in zip(got, good))
+
+
+def test_decode_route_with_default_metadata(gpu):
+    # compute_mask_kernel packs PARTIAL tiles by default; sparse_attention with fewer than 32 query rows must still
+    # reach the split-KV kernels (which read the bool mask) with that metadata
+    B, H, Sq, Sk, D, BK = 2, 2, 8, 1024, 64, 32
+    q, k, v = W.qkv(B, H, Sq, D, torch.bfloat16, seed=13, device=gpu, Sk=Sk)
+    mask = (torch.rand(Sq, Sk, generator=torch.Generator().manual_seed(14)) < 0.3).to(gpu)
+    mask[:, :BK] = True
+    me = mask[None, None].expand(B, H, Sq, Sk)
+    md = compute_mask_kernel(me, Sq, BK)
+    assert md.packed_masks is not None
+    o = sparse_attention(q, k, v, me, Sq, BK, md)
+    assert torch.equal(o, sparse_attention_decode(q, k, v, me, BK, md))
+    assert (o.float() - sdpa32(q, k, v, mask)).abs().max() <= TOL
+    md2 = compute_mask_kernel(me, Sq, BK, schedule=None, pack_partial=False)
+    assert torch.equal(o, sparse_attention(q, k, v, me, Sq, BK, md2))
+    with pytest.raises(ValueError, match="mask"):
+        sparse_attention(q, k, v, None, Sq, BK, md)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_cpu_plumbing_workload_on_the_gpu(gpu, dtype):
+    # B=1 H=4 S=512 D=64, q/k/v ~ N(0,1) from seed 0 in fp32, mask: 32x32 blocks empty w.p. 0.5, 10 % of the blocks
+    # coin flips, diagonal True.  Lists bit-exact against the oracle; the fp32 inputs cast to the kernel's dtypes against
+    # fp32 masked SDPA of the fp32 inputs.
+    B, H, S, D = 1, 4, 512, 64
+    q32, k32, v32 = W.qkv(B, H, S, D, torch.float32, seed=0)
+    mask = W.random_block_mask(S, 32, 0.5, seed=0)
+    want = F.scaled_dot_product_attention(q32, k32, v32, attn_mask=mask)
+    q, k, v = (t.to(gpu, dtype) for t in (q32, k32, v32))
+    me = mask.to(gpu)[None, None].expand(B, H, S, S)
+    for BQ, BK in ((32, 32), (128, 32), (64, 64)):
+        md = compute_mask_kernel(me, BQ, BK)
+        assert_metadata_equal(md, oracle.classify(mask.numpy()[None, None].repeat(H, 1), BQ, BK), f"{BQ}x{BK}")
+        o = sparse_attention(q, k, v, me, BQ, BK, md)
+        assert (o.float().cpu() - want).abs().max() <= TOL
+    with pytest.raises(TypeError, match="float32"):
+        sparse_attention(q32.to(gpu), k32.to(gpu), v32.to(gpu), me, 32, 32)
