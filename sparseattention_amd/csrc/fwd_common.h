@@ -115,6 +115,41 @@ __device__ __forceinline__ void dma16(const void *base, uint32_t lane_offset, ui
         : "memory");  // m0 is written; nothing else in these kernels keeps a value in it
 }
 
+// N dwords from N wave-uniform addresses by scalar loads that are issued back to back and share ONE wait.  Left to
+// the compiler, loads whose addresses it forms one after the other are waited for one after the other as well, a
+// memory round trip each; at the start of a Q tile that is most of the time before the first K/V request.
+template <int N>
+__device__ __forceinline__ void scalar_gather(const int32_t *const (&a)[N], int (&o)[N]) {
+    static_assert(N == 4 || N == 6 || N == 10, "counts + first slots of both lists for 1, 2 or 4 entries per chunk");
+    const uint64_t *const q = reinterpret_cast<const uint64_t *>(&a[0]);  // (pointers as 64-bit scalars)
+    if constexpr (N == 4) {
+        asm volatile(
+            "s_load_dword %0, %4, 0x0\n\ts_load_dword %1, %5, 0x0\n\ts_load_dword %2, %6, 0x0\n\t"
+            "s_load_dword %3, %7, 0x0\n\ts_waitcnt lgkmcnt(0)"
+            : "=&s"(o[0]), "=&s"(o[1]), "=&s"(o[2]), "=&s"(o[3])
+            : "s"(q[0]), "s"(q[1]), "s"(q[2]), "s"(q[3])
+            : "memory");
+    } else if constexpr (N == 6) {
+        asm volatile(
+            "s_load_dword %0, %6, 0x0\n\ts_load_dword %1, %7, 0x0\n\ts_load_dword %2, %8, 0x0\n\t"
+            "s_load_dword %3, %9, 0x0\n\ts_load_dword %4, %10, 0x0\n\ts_load_dword %5, %11, 0x0\n\t"
+            "s_waitcnt lgkmcnt(0)"
+            : "=&s"(o[0]), "=&s"(o[1]), "=&s"(o[2]), "=&s"(o[3]), "=&s"(o[4]), "=&s"(o[5])
+            : "s"(q[0]), "s"(q[1]), "s"(q[2]), "s"(q[3]), "s"(q[4]), "s"(q[5])
+            : "memory");
+    } else {
+        asm volatile(
+            "s_load_dword %0, %10, 0x0\n\ts_load_dword %1, %11, 0x0\n\ts_load_dword %2, %12, 0x0\n\t"
+            "s_load_dword %3, %13, 0x0\n\ts_load_dword %4, %14, 0x0\n\ts_load_dword %5, %15, 0x0\n\t"
+            "s_load_dword %6, %16, 0x0\n\ts_load_dword %7, %17, 0x0\n\ts_load_dword %8, %18, 0x0\n\t"
+            "s_load_dword %9, %19, 0x0\n\ts_waitcnt lgkmcnt(0)"
+            : "=&s"(o[0]), "=&s"(o[1]), "=&s"(o[2]), "=&s"(o[3]), "=&s"(o[4]), "=&s"(o[5]), "=&s"(o[6]), "=&s"(o[7]),
+              "=&s"(o[8]), "=&s"(o[9])
+            : "s"(q[0]), "s"(q[1]), "s"(q[2]), "s"(q[3]), "s"(q[4]), "s"(q[5]), "s"(q[6]), "s"(q[7]), "s"(q[8]), "s"(q[9])
+            : "memory");
+    }
+}
+
 // Swizzles of the 16-byte pieces inside an LDS row.  Rows are stored unpadded (D*2 bytes) because a
 // direct global->LDS load writes 64 lanes x 16 bytes contiguously; instead the piece index is XORed
 // with a function of the row so that

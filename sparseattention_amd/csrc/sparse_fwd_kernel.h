@@ -103,6 +103,9 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
     // this lane's row in a packed tile: BK/8 bytes per row, NW*32 rows per tile
     const int64_t tile_bytes = (int64_t)(NW * 4) * p.BK;
     const int sh4 = 4 * hh;
+    // (see the loads next to the counts below)
+    constexpr bool kEarlyFirstChunk = !PS && !PP && D <= 128;  // (at D = 256 the registers are all taken)
+    int early_f[EPC] = {}, early_p[EPC] = {};
     // what load_mask needs to know of a Q tile
     struct MaskSrc {
         const uint8_t *mrow, *prow;
@@ -149,6 +152,21 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
         orow_off = b * p.os[0] + h * p.os[1] + (int64_t)qrow_ * p.os[2] + 4 * hh;
         lse_off = b * p.lses[0] + h * p.lses[1] + (int64_t)qrow_ * p.lses[2];
     };
+    // Q^T operand: lane (l32, hh) keeps d = 16c + 8hh .. +7 of its query row for every 16-wide step c.
+    u32x4 qf[D / 16];
+    auto load_q = [&](int b_, int h_, int qt_) {
+        const int qrow_ = qt_ * (NW * 32) + wave * 32 + l32;
+        const uint16_t *qp = p.q + b_ * p.qs[0] + h_ * p.qs[1] + (int64_t)qrow_ * p.qs[2] + 8 * hh;
+#pragma unroll
+        for (int c = 0; c < D / 16; c++) qf[c] = *(const u32x4 *)(qp + 16 * c);
+    };
+    // The scale (softmax scale / ln 2) goes into Q once, so that the S MFMAs deliver exp2 arguments.
+    auto scale_q = [&]() {
+#pragma unroll
+        for (int c = 0; c < D / 16; c++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) qf[c][e] = E::scale2(qf[c][e], p.scale);
+    };
     // Row of this workgroup in the schedule: entry 0 = {number of Q tiles, -, -, -}, then one entry
     // {(b << 16) | h, qt, F, P} per Q tile.
     const int4 *const sched_row = reinterpret_cast<const int4 *>(p.sched) + (int64_t)blockIdx.x * (p.sched_R + 1);
@@ -169,27 +187,43 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
         const int bh = 2 * pair + (paired ? (r & 1) : 0);
         const int qt0 = p.nQ - 1 - (paired ? (r >> 1) : r);
         const int b0 = bh / p.H, h0 = bh - b0 * p.H;
-        set_item(b0, h0, qt0, p.full_lens[b0 * p.fls[0] + h0 * p.fls[1] + qt0 * p.fls[2]],
-                 p.part_lens[b0 * p.pls[0] + h0 * p.pls[1] + qt0 * p.pls[2]]);
+        // The queries come from HBM, the longest wait of a tile's start: requested first of all.  Then the counts and,
+        // with them, the first slots of both lists (uniform addresses: scalar loads under one wait), so that the first
+        // K/V chunk can be requested one memory round trip earlier, before the list has made its way to LDS.  Slots
+        // past a count hold anything; early_entry() picks the ones that count.
+        const int32_t *const fl0 = p.full_lens + (b0 * p.fls[0] + h0 * p.fls[1] + qt0 * p.fls[2]);
+        const int32_t *const pl0 = p.part_lens + (b0 * p.pls[0] + h0 * p.pls[1] + qt0 * p.pls[2]);
+        if constexpr (kEarlyFirstChunk) {
+            load_q(b0, h0, qt0);
+            const int32_t *f0 = p.full_ids + b0 * p.fis[0] + h0 * p.fis[1] + qt0 * p.fis[2];
+            const int32_t *p0 = p.part_ids + b0 * p.pis[0] + h0 * p.pis[1] + qt0 * p.pis[2];
+            const int32_t *addr[2 + 2 * EPC];
+            int got[2 + 2 * EPC];
+            addr[0] = fl0;
+            addr[1] = pl0;
+            static_for<EPC>([&](auto i_c) {
+                constexpr int i = decltype(i_c)::value;
+                const int slot = i < p.nK ? i : p.nK - 1;  // (a row of fewer than EPC tiles: stay inside it)
+                addr[2 + i] = f0 + (int64_t)slot * p.fis[3];
+                addr[2 + EPC + i] = p0 + (int64_t)slot * p.pis[3];
+            });
+            scalar_gather(addr, got);
+            static_for<EPC>([&](auto i_c) {
+                constexpr int i = decltype(i_c)::value;
+                early_f[i] = got[2 + i];
+                early_p[i] = got[2 + EPC + i];
+            });
+            set_item(b0, h0, qt0, got[0], got[1]);
+        } else {
+            set_item(b0, h0, qt0, *fl0, *pl0);
+        }
     }
 
-    // Q^T operand: lane (l32, hh) keeps d = 16c + 8hh .. +7 of its query row for every 16-wide step c.
-    u32x4 qf[D / 16];
-    auto load_q = [&](int b_, int h_, int qt_) {
-        const int qrow_ = qt_ * (NW * 32) + wave * 32 + l32;
-        const uint16_t *qp = p.q + b_ * p.qs[0] + h_ * p.qs[1] + (int64_t)qrow_ * p.qs[2] + 8 * hh;
-#pragma unroll
-        for (int c = 0; c < D / 16; c++) qf[c] = *(const u32x4 *)(qp + 16 * c);
-    };
-    // The scale (softmax scale / ln 2) goes into Q once, so that the S MFMAs deliver exp2 arguments.
-    auto scale_q = [&]() {
-#pragma unroll
-        for (int c = 0; c < D / 16; c++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) qf[c][e] = E::scale2(qf[c][e], p.scale);
-    };
-    load_q(b, h, qt);
-    scale_q();
+    // (the plain loop requests its first K/V chunk and its list before its queries, see there)
+    if constexpr (!kEarlyFirstChunk) {
+        load_q(b, h, qt);
+        scale_q();
+    }
 
     // Online-softmax state of this lane's query row.  Exponentials are taken against a reference value m_ref
     // (exp2 units).  The S MFMAs start from the accumulator -m_ref (neg_m: the same value in all 16 registers,
@@ -260,15 +294,40 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
     constexpr int kAbsent = (int)0x80000000u;
     const int list_cnt = MODE == 2 ? NE : (NE + EPC - 1) / EPC * EPC;
     const bool list_in_lds = !PS && list_cnt <= kListCap;
+    // (the strides as scalars, read here: left inside the lane-dependent branch below they are fetched from the
+    // argument block by a vector load of their own, a memory round trip in front of every list load)
+    int64_t fis3 = p.fis[3], pis3 = p.pis[3];
+    asm volatile("" : "+s"(fis3), "+s"(pis3));
     auto tagged_entry = [&](int e) -> int {  // from global memory
         if (e >= NE) return kAbsent;
-        const int idx = e < F ? fid[(int64_t)e * p.fis[3]] : pid[(int64_t)(e - F) * p.pis[3]];
+        const int idx = e < F ? fid[(int64_t)e * fis3] : pid[(int64_t)(e - F) * pis3];
         if ((unsigned)idx >= (unsigned)p.nK) return kAbsent;
         return (MODE == 2 ? (idx << p.lbk) : (idx << LBKC)) | (e >= F ? kPartialBit : 0);
     };
-    if (list_in_lds) {
-        for (int e = tid; e < list_cnt; e += NW * 64) ent[e] = tagged_entry(e);
-    }
+    // list slot E of the tile's first chunk, from the slots that came with the counts, tagged like an LDS entry
+    auto early_entry = [&](auto e_c) -> int {
+        constexpr int e = decltype(e_c)::value;
+        if (e >= NE) return kAbsent;
+        int idx = early_f[e];
+        if (e >= F) {
+            idx = early_p[0];
+            static_for<e>([&](auto j_c) {  // e - F is one of 0 .. e
+                constexpr int j = decltype(j_c)::value + 1;
+                // (a value that passed through an asm statement is no array element any more: the compiler would
+                // otherwise fold this chain of selects into one load at a variable index, from scratch memory)
+                int cand = __builtin_amdgcn_readfirstlane(early_p[j]);
+                asm volatile("" : "+s"(cand));
+                if (e - F == j) idx = cand;
+            });
+        }
+        if ((unsigned)idx >= (unsigned)p.nK) return kAbsent;
+        return (MODE == 2 ? (idx << p.lbk) : (idx << LBKC)) | (e >= F ? kPartialBit : 0);
+    };
+    auto copy_list = [&]() {
+        if (list_in_lds) {
+            for (int e = tid; e < list_cnt; e += NW * 64) ent[e] = tagged_entry(e);
+        }
+    };
     // First key column of every list entry in chunk t (t < T), plus which entries exist / are partial, in two
     // steps: entries_read issues the reads of the list (the values are the same in all lanes), entries_use turns
     // them into scalars.  The main loop reads the entries of a chunk one iteration before it needs them, so
@@ -567,8 +626,13 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) s[kb][i] -= delta;
+            // (= -m_ref either way; formed in place the sixteen registers need no copy on the path that does not raise,
+            // but at D = 256, where every register is taken, that form spills)
 #pragma unroll
-            for (int i = 0; i < 16; i++) neg_m[i] = -m_ref;
+            for (int i = 0; i < 16; i++) {
+                if constexpr (D <= 128) neg_m[i] -= delta;
+                else neg_m[i] = -m_ref;
+            }
 #pragma unroll
             for (int i = 0; i < 2; i++) acc_l[i] *= a;  // the lane only ever reads the one of its own row
 #pragma unroll
@@ -881,6 +945,7 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
             unsigned vl[2] = {0u, 0u}, pt[2] = {0u, 0u};
             constexpr unsigned ALL = (1u << EPC) - 1u;
             constexpr int kOpsPerChunk = 2 * NLD;
+            copy_list();
             __syncthreads();  // the list in LDS is complete
             chunk_entries(0, col, valid, part);
             stage_chunk(0, col);
@@ -946,9 +1011,30 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
         unsigned vl[2] = {0u, 0u}, pt[2] = {0u, 0u};
         constexpr unsigned ALL = (1u << EPC) - 1u;
         StagePlan pl;  // where the chunk fetched by the current iteration comes from
+        // The first chunk is requested from the list slots that came with the counts, before the list itself is
+        // copied (its loads would otherwise have to land first: one memory round trip per Q tile).
+        if constexpr (kEarlyFirstChunk) {
+            // The queries were requested first of all; now the first K/V chunk, then the list.
+            int raw0[EPC];
+            static_for<EPC>([&](auto j_c) { raw0[decltype(j_c)::value] = early_entry(j_c); });
+            entries_use(0, raw0, col, valid, part);
+            stage_chunk(0, col);
+            const bool mine = list_in_lds && tid < list_cnt;
+            int first_slots = 0;
+            if (mine) first_slots = tagged_entry(tid);
+            if (mine) ent[tid] = first_slots;
+            if (list_in_lds)
+                for (int e = tid + NW * 64; e < list_cnt; e += NW * 64) ent[e] = tagged_entry(e);
+        } else {
+            copy_list();
+        }
         __syncthreads();  // the list in LDS is complete
-        chunk_entries(0, col, valid, part);
-        stage_chunk(0, col);
+        if constexpr (kEarlyFirstChunk) {
+            scale_q();
+        } else {
+            chunk_entries(0, col, valid, part);
+            stage_chunk(0, col);
+        }
         sp[0] = part != 0u || valid != ALL;
         vl[0] = valid;
         pt[0] = part;
