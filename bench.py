@@ -20,7 +20,11 @@ the reference also excludes preprocessing from the forward time and reports it s
   backward   dq, dk, dv of the headline workload (sparse_attention_backward) against the MFMA peak
   decode     the split-KV kernels for few query rows (sparse_attention_decode) against the HBM peak: K and V of
              the executed tiles are read once
-  cpu_baseline / cpu_sdpa_baseline   the CPU oracle and torch's masked SDPA on a bounded sample
+  configs    the forward on the two long-sequence configurations (documents B4 H32 S16384, composed B1 H32 S32768),
+             each with its own roofline against the MFMA peak
+  tile_selection   every candidate tile size of select_block_sizes timed on four masks, next to what it picked
+  cpu_baseline     torch's masked SDPA on CPU tensors of the whole workload: the reference's own check path
+                   (test_attn.py:40) on the host cores; cpu_oracle_baseline: the C oracle (a port) on the same workload
 """
 import argparse
 import gc
@@ -47,6 +51,14 @@ TRAFFIC_DECODE_BYTES = (4.2959e9, 1.6225e9)
 # 4242 MiB read + 776 MiB written
 TRAFFIC_BWD_CAUSAL_BYTES = 5.262e9
 
+# where the constants above come from (refreshed whenever a kernel changes: same commands as in the files)
+TRAFFIC_SOURCE = {
+    "forward": "profiles/sparse_fwd_kernel_causal_B8H32S4096D128.txt section 2",
+    "mask_classify": "profiles/mask_classify_kernels_mask_32768x32768.txt section 2",
+    "decode": "profiles/sparse_decode_kernel_B8H32Sk32768D128.txt",
+    "backward": "profiles/sparse_bwd_kernel_causal_B8H32S4096D128.txt",
+}
+
 SETTLE_LAUNCHES = 30
 
 B, H, S, D = 8, 32, 4096, 128
@@ -64,6 +76,8 @@ def parse():
     ap.add_argument("--no-classify", action="store_true", help="skip the mask-classification timing")
     ap.add_argument("--no-decode", action="store_true", help="skip the few-query-rows (decode) timing")
     ap.add_argument("--no-backward", action="store_true", help="skip the backward-pass timing")
+    ap.add_argument("--no-long", action="store_true", help="skip the forward on the documents and composed configurations")
+    ap.add_argument("--no-tiles", action="store_true", help="skip the timing of the tile-size candidates")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy a few times, so that a counter run over this command "
                          "holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -103,22 +117,25 @@ def time_launches(fn, steps, warmup):
     return wall_ms, ev_ms
 
 
-def forward_case(name, mask2d, q, k, v, steps, warmup, schedule=None, pack_partial=None, block_k=BK):
+def forward_case(name, mask2d, q, k, v, steps, warmup, schedule=None, pack_partial=None, block_k=BK, block_q=BQ):
     import torch
     from sparseattention_amd import compute_mask_kernel, sparse_attention
 
+    B, H, S, D = q.shape
+    BQ = block_q
     me = mask2d[None, None].expand(B, H, S, S)
     md = compute_mask_kernel(me, BQ, block_k, pack_partial=pack_partial, schedule=schedule)
     tiles_plane = int(md.unmasked_lens[0, 0].sum()) + int(md.masked_lens[0, 0].sum())
     partial_plane = int(md.masked_lens[0, 0].sum())
-    frac = float(mask2d.float().mean())
+    # mean of the mask in row slabs (a [32768,32768] float copy would take 4 GiB)
+    frac = sum(float(mask2d[r0:r0 + 2048].sum()) for r0 in range(0, S, 2048)) / (S * S)
     wall_ms, ev_ms = time_launches(lambda: sparse_attention(q, k, v, me, BQ, block_k, mask_metadata=md), steps, warmup)
     executed = tiles_plane * B * H * 4 * BQ * block_k * D
     useful = 4 * B * H * S * S * D * frac
     return {
         "mask": name,
         "fraction_unmasked": round(frac, 5),
-        "executed_tile_fraction": round(tiles_plane / ((S // BQ) * (S // BK)), 5),
+        "executed_tile_fraction": round(tiles_plane / ((S // BQ) * (S // block_k)), 5),
         "partial_tiles_per_plane": partial_plane,
         "ms": round(wall_ms, 4),
         "kernel_ms": round(ev_ms, 4),
@@ -171,7 +188,8 @@ def classify_case(steps, warmup):
         "pack_partial_ms": round(pack_ms, 4),
         "roofline": {"bound": "hbm", "achieved": round(nbytes / (ev_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(nbytes / (ev_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-                     "traffic": TRAFFIC_CLASSIFY_1GIB_BYTES, "algorithmic_bytes": nbytes},
+                     "traffic": TRAFFIC_CLASSIFY_1GIB_BYTES, "traffic_source": TRAFFIC_SOURCE["mask_classify"],
+                     "algorithmic_bytes": nbytes},
     }
 
 
@@ -233,6 +251,7 @@ def backward_case(q, k, v, steps, warmup):
         "executed_tflops": round(executed / (ev_ms * 1e-3) / 1e12, 1),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BWD_CAUSAL_BYTES,
+                     "traffic_source": TRAFFIC_SOURCE["backward"],
                      "kernel": "sparse_bwd_kernel x3 (+ bwd_prepare_kernel)", "flop_per_launch": algorithmic},
     }
 
@@ -269,15 +288,79 @@ def decode_case(steps, warmup):
             "ms": round(wall_ms, 4), "kernel_ms": round(ev_ms, 4),
             "roofline": {"bound": "hbm", "achieved": round(nbytes / (ev_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
                          "unit": "GB/s", "frac": round(nbytes / (ev_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-                         "traffic": TRAFFIC_DECODE_BYTES[case], "algorithmic_bytes": nbytes,
+                         "traffic": TRAFFIC_DECODE_BYTES[case], "traffic_source": TRAFFIC_SOURCE["decode"],
+                         "algorithmic_bytes": nbytes,
                          "kernel": "sparse_decode_kernel (+ decode_merge_kernel)"},
         })
     return rows
 
 
+def long_configs(steps, warmup):
+    """The forward on configs[3] (documents) and configs[4] (composed): tiles 128x32, packed partial tiles, metadata
+    precomputed; executed-tile flop against the MFMA peak."""
+    import torch
+    from sparseattention_amd import workloads as W
+
+    rows = []
+    for name, Bc, Hc, Sc, make in (
+            ("configs[3]: documents, B=4 H=32 S=16384 D=128 bf16; doc lengths uniform in [256,4096], causal within a document; "
+             "bool mask [16384,16384] (256 MiB) shared by all planes", 4, 32, 16384, lambda: W.document_mask(16384, seed=0, device="cuda")),
+            ("configs[4]: composed, B=1 H=32 S=32768 D=128 bf16; (kv<=q and q-kv<1024) or (q<2048 and kv<2048); bool mask "
+             "[32768,32768] (1 GiB) shared by all heads", 1, 32, 32768, lambda: W.composed_mask(32768, device="cuda"))):
+        q, k, v = W.qkv(Bc, Hc, Sc, D, torch.bfloat16, seed=0, device="cuda")
+        mask = make()
+        r = forward_case(name, mask, q, k, v, steps, warmup)
+        achieved = r["_executed_flop"] / (r["kernel_ms"] * 1e-3) / 1e12
+        rows.append({
+            "workload": name + "; tiles BLOCK_Q=128 BLOCK_K=32",
+            "fraction_unmasked": r["fraction_unmasked"], "executed_tile_fraction": r["executed_tile_fraction"],
+            "executed_tiles_per_plane": int(r["_executed_flop"] // (Bc * Hc * FLOP_PER_TILE)),
+            "partial_tiles_per_plane": r["partial_tiles_per_plane"],
+            "ms": r["ms"], "kernel_ms": r["kernel_ms"], "effective_tflops": r["effective_tflops"],
+            "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": "sparse_fwd_kernel",
+                         "flop_per_launch": r["_executed_flop"]},
+        })
+        del q, k, v, mask
+        torch.cuda.empty_cache()
+    return rows
+
+
+def tile_selection_case(steps, warmup):
+    """select_block_sizes against the clock: every candidate tile size is classified and timed on four masks (the
+    forward at B=2 H=32 D=128 bf16, so that the large masks fit beside q, k, v), next to the candidate the cost model
+    picks.  `regret` = time of the pick / best measured time - 1."""
+    import torch
+    from sparseattention_amd import (compute_mask_kernel, select_block_sizes, sparse_attention, workloads as W)
+    from sparseattention_amd.mask_utils import DEFAULT_TILE_CANDIDATES
+
+    out = []
+    for name, Sc, make in (("causal S=4096", 4096, lambda: W.causal_mask(4096, "cuda")),
+                           ("random blocks p=0.75 S=4096", 4096, lambda: W.random_block_mask(4096, 128, 0.75, seed=75, device="cuda")),
+                           ("documents S=16384", 16384, lambda: W.document_mask(16384, seed=0, device="cuda")),
+                           ("composed S=32768", 32768, lambda: W.composed_mask(32768, device="cuda"))):
+        Bc, Hc = (2, 32) if Sc <= 16384 else (1, 32)
+        q, k, v = W.qkv(Bc, Hc, Sc, D, torch.bfloat16, seed=0, device="cuda")
+        me = make()[None, None].expand(Bc, Hc, Sc, Sc)
+        pick_q, pick_k, _, report = select_block_sizes(me)
+        timed = {}
+        for bq, bk in DEFAULT_TILE_CANDIDATES:
+            md = compute_mask_kernel(me, bq, bk)
+            _, ev = time_launches(lambda: sparse_attention(q, k, v, me, bq, bk, mask_metadata=md), steps, warmup)
+            timed[f"{bq}x{bk}"] = round(ev, 4)
+            del md
+        best = min(timed, key=timed.get)
+        out.append({"mask": name, "B": Bc, "H": Hc, "picked": f"{pick_q}x{pick_k}", "best_measured": best,
+                    "regret": round(timed[f"{pick_q}x{pick_k}"] / timed[best] - 1.0, 4), "kernel_ms": timed,
+                    "model_cost": {f"{r[0]}x{r[1]}": round(r[4] / 1e6, 2) for r in report}})
+        del q, k, v, me
+        torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baselines():
-    """Bounded CPU legs on the host cores: (a) the C oracle (a port of the reference algorithm),
-    (b) torch's masked SDPA on CPU tensors, the reference's own check path (test_attn.py:40)."""
+    """Bounded CPU legs on the host cores: cpu_baseline = torch's masked SDPA on CPU tensors, the reference's own CPU
+    path (test_attn.py:40); cpu_oracle_baseline = the C oracle (a port of the reference algorithm)."""
     import torch
     import torch.nn.functional as F
 
@@ -297,7 +380,7 @@ def cpu_baselines():
     oracle.forward(qf, kf, vf, m4, BQ, BK, meta=meta, p_round=1)
     dt = time.perf_counter() - t0
     useful = 4 * 1 * hp * S * S * D * frac
-    out["cpu_baseline"] = {
+    out["cpu_oracle_baseline"] = {
         "value": round(useful / dt / 1e12, 5), "unit": "TFLOP/s", "cores": oracle.max_threads(), "kind": "port",
         "sample": f"C oracle two-pass forward (oracle/sparse_oracle.c, OpenMP) on all {hp} (b,h) planes of the workload "
                   f"(causal S={S} D={D}, bf16 inputs widened to fp32, tiles {BQ}x{BK}): {dt:.2f} s, effective TFLOP/s",
@@ -315,10 +398,12 @@ def cpu_baselines():
         ts.append(time.perf_counter() - t0)
     dt = sorted(ts)[1]
     useful = 4 * 1 * hs * S * S * D * frac
-    out["cpu_sdpa_baseline"] = {
-        "value": round(useful / dt / 1e12, 5), "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "library",
-        "sample": f"torch {torch.__version__} F.scaled_dot_product_attention(q,k,v,attn_mask=mask) on CPU bf16 tensors, "
-                  f"all {hs} (b,h) planes of the workload, median of 3: {dt:.3f} s, effective TFLOP/s",
+    out["cpu_baseline"] = {
+        "value": round(useful / dt / 1e12, 5), "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "reference",
+        "sample": f"the reference's CPU path for this workload is one library call, torch {torch.__version__} "
+                  f"F.scaled_dot_product_attention(q,k,v,attn_mask=mask) (test_attn.py:40; none of the reference's own "
+                  f"code runs): CPU bf16 tensors, all {hs} (b,h) planes of the workload (causal S={S} D={D}), one "
+                  f"warm-up, median of 3 passes: {dt:.3f} s, effective TFLOP/s",
         "ms_full_workload": round(dt * 1e3 * B * H / hs, 1),
         "host_cpu_count": os.cpu_count(),
     }
@@ -351,6 +436,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_launches": max(0, SETTLE_LAUNCHES - args.warmup),  # untimed launches in front of the warm-up
         "ms_per_step": head["ms"],
         "higher_is_better": True,
         "scaling": "weak",
@@ -364,6 +450,7 @@ def main():
                    "partial_tiles_per_plane": head["partial_tiles_per_plane"]},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_FWD_CAUSAL_BYTES,
+                     "traffic_source": TRAFFIC_SOURCE["forward"],
                      "kernel": "sparse_fwd_kernel", "kernel_ms": head["kernel_ms"],
                      "flop_per_launch": head["_executed_flop"]},
     }
@@ -395,6 +482,11 @@ def main():
     if not args.no_backward:
         result["backward"] = backward_case(q, k, v, max(10, args.steps // 5), max(5, args.warmup // 2))
     del q, k, v
+    torch.cuda.empty_cache()
+    if not args.no_long:
+        result["configs"] = long_configs(max(20, args.steps // 2), max(10, args.warmup))
+    if not args.no_tiles:
+        result["tile_selection"] = tile_selection_case(max(10, args.steps // 5), max(10, args.warmup // 2))
     if not args.no_decode:
         result["decode"] = decode_case(max(20, args.steps // 2), max(10, args.warmup))
     if args.calibrate_copy:

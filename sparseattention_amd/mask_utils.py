@@ -182,11 +182,20 @@ def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int, pack_par
     return md
 
 
-# Tile sizes tried by select_block_sizes, and what one executed mask entry costs at each BLOCK_Q relative to
-# BLOCK_Q = 128 (measured on MI355X with every tile executed, B8 H32 S4096 D128 bf16; BLOCK_K does not enter:
-# the forward consumes keys in chunks of 64 whatever the tile width).
+# Tile sizes tried by select_block_sizes, and what one executed mask entry costs at each of them relative to tiles of
+# 128 x 64 (measured on MI355X, D = 128 bf16, with bench.py's tile_selection leg: the same mask classified and run at
+# every candidate; causal S=4096, random blocks p=0.75, documents S=16384 and the composed mask S=32768 agree within
+# 3 %).  BLOCK_Q sets most of it (rows per workgroup: 64-row tiles fetch K/V twice as often per entry, 256-row tiles
+# run the two-phase kernel); BLOCK_K only through the scalar bookkeeping per list entry (the forward consumes keys in
+# chunks of 64 whatever the tile width).
 DEFAULT_TILE_CANDIDATES = ((128, 32), (128, 64), (128, 128), (64, 32), (64, 64), (256, 32), (256, 64))
-RELATIVE_COST_PER_ENTRY = {32: 1.55, 64: 1.2, 128: 1.0, 256: 1.05}
+RELATIVE_COST_PER_ENTRY = {32: 2.0, 64: 1.45, 128: 1.0, 256: 1.1}
+RELATIVE_COST_BLOCK_K = {16: 1.08, 32: 1.03, 64: 1.0}  # wider tiles: 1.005
+
+
+def entry_cost(BLOCK_Q: int, BLOCK_K: int) -> float:
+    """Relative cost of one executed mask entry at these tile sizes (see the tables above)."""
+    return RELATIVE_COST_PER_ENTRY.get(BLOCK_Q, 1.0) * RELATIVE_COST_BLOCK_K.get(BLOCK_K, 1.005)
 
 
 def select_block_sizes(mask: torch.Tensor, candidates=DEFAULT_TILE_CANDIDATES, partial_cost: float = 1.25):
@@ -196,7 +205,7 @@ def select_block_sizes(mask: torch.Tensor, candidates=DEFAULT_TILE_CANDIDATES, p
     masked-out blocks", README.md:64).  Every candidate (BLOCK_Q, BLOCK_K) that divides the mask is
     classified (on the GPU when the mask lives there, else with compute_mask_slow) and priced as
 
-        (full tiles + partial_cost * partial tiles) * BLOCK_Q * BLOCK_K * RELATIVE_COST_PER_ENTRY[BLOCK_Q]
+        (full tiles + partial_cost * partial tiles) * BLOCK_Q * BLOCK_K * entry_cost(BLOCK_Q, BLOCK_K)
 
     summed over the distinct mask planes; partial tiles cost more because their mask is read and applied.
     Returns ``(BLOCK_Q, BLOCK_K, metadata, report)``: the cheapest candidate, its MaskMetadata (ready to pass
@@ -215,7 +224,7 @@ def select_block_sizes(mask: torch.Tensor, candidates=DEFAULT_TILE_CANDIDATES, p
         # broadcast planes hold the same counts: the sum over the expanded view weights every plane equally
         full = int(md.unmasked_lens.sum())
         part = int(md.masked_lens.sum())
-        cost = (full + partial_cost * part) * BQ * BK * RELATIVE_COST_PER_ENTRY.get(BQ, 1.0)
+        cost = (full + partial_cost * part) * BQ * BK * entry_cost(BQ, BK)
         report.append((BQ, BK, full, part, cost))
         if best is None or cost < best[0]:
             best = (cost, BQ, BK, md)
