@@ -43,7 +43,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E peak, GB/s
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this script and scaled by
 # the readings of a 1 GiB device copy in the same run (--calibrate-copy).  The summaries with the commands
 # are profiles/sparse_fwd_kernel_causal_B8H32S4096D128.txt and profiles/mask_classify_kernels_mask_32768x32768.txt.
-TRAFFIC_FWD_CAUSAL_BYTES = 1.3070e9      # 990.1 MiB read + 256.3 MiB written
+TRAFFIC_FWD_CAUSAL_BYTES = 1.1708e9      # 860.6 MiB read + 256.0 MiB written
 TRAFFIC_CLASSIFY_1GIB_BYTES = 1.0744e9   # 1,048,622 + 327 KiB read, 256 + 45.5 KiB written
 # decode workloads (profiles/sparse_decode_kernel_B8H32Sk32768D128.txt), both kernels
 TRAFFIC_DECODE_BYTES = (4.2959e9, 1.6225e9)
