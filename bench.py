@@ -60,6 +60,7 @@ TRAFFIC_SOURCE = {
 }
 
 SETTLE_LAUNCHES = 30
+SETTLE_MS = 40.0
 
 B, H, S, D = 8, 32, 4096, 128
 BQ, BK = 128, 32
@@ -101,6 +102,14 @@ def time_launches(fn, steps, warmup):
         # untimed launches go in front of it
         for _ in range(max(0, SETTLE_LAUNCHES - warmup)):
             fn()
+        # ... and by time as well: after seconds of host work (a mask built on the CPU) the device sits in a low power
+        # state, from which short kernels need tens of milliseconds of load to come back
+        torch.cuda.synchronize()
+        t_settle = time.perf_counter()
+        while (time.perf_counter() - t_settle) * 1e3 < SETTLE_MS:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
@@ -436,7 +445,8 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "settle_launches": max(0, SETTLE_LAUNCHES - args.warmup),  # untimed launches in front of the warm-up
+        # untimed launches in front of the warm-up: this many, then more until settle_ms of load have passed
+        "settle_launches": max(0, SETTLE_LAUNCHES - args.warmup), "settle_ms": SETTLE_MS,
         "ms_per_step": head["ms"],
         "higher_is_better": True,
         "scaling": "weak",

@@ -88,7 +88,7 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
     const int l32 = lane & 31, hh = lane >> 5;
 
     // Workgroup -> (b, h, Q tile).  Hardware hands consecutive workgroup ids to the 8 XCDs in turn; the
-    // remap gives each XCD a contiguous range of the (b,h)-major order so that the Q tiles sharing one
+    // remap gives each XCD whole planes (every eighth pair of the (b,h)-major order) so that the Q tiles sharing one
     // K/V plane run on the XCD whose L2 already holds it.  Planes are taken two at a time with their Q tiles
     // interleaved, last Q tile first (under causal-like masks it has the longest list): the slots that finish
     // the short tiles of one pair then pick up the long tiles of the next, which evens out the load.
@@ -182,7 +182,16 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
         const int total = gridDim.x, per = total >> 3;
         int lin = blockIdx.x;
         if (lin < (per << 3)) lin = (lin & 7) * per + (lin >> 3);
-        const int pair = lin / (2 * p.nQ), r = lin - pair * 2 * p.nQ;
+        int pair = lin / (2 * p.nQ);
+        const int r = lin - pair * 2 * p.nQ;
+        // Which pairs of planes an XCD gets: every eighth one, so that a mask that differs between batch elements
+        // (whose planes are neighbours in this order) loads the XCDs alike; a contiguous range when the pairs do
+        // not divide evenly.
+        if (((p.B * p.H) & 15) == 0) {
+            const int ppx = (p.B * p.H) >> 4;  // pairs per XCD
+            const int x = pair / ppx;
+            pair = (pair - x * ppx) * 8 + x;
+        }
         const bool paired = 2 * pair + 1 < p.B * p.H;  // the last plane of an odd count goes alone
         const int bh = 2 * pair + (paired ? (r & 1) : 0);
         const int qt0 = p.nQ - 1 - (paired ? (r >> 1) : r);

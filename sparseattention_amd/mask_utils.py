@@ -233,6 +233,59 @@ def select_block_sizes(mask: torch.Tensor, candidates=DEFAULT_TILE_CANDIDATES, p
     return best[1], best[2], best[3], report
 
 
+@dataclass
+class Tiling:
+    """A choice of tile sizes and of the tile grid's origin for one mask (:func:`select_tiling`).
+
+    The grid of BLOCK_Q x BLOCK_K tiles starts ``q_offset`` rows above and ``k_offset`` columns left of the mask's
+    first entry: the mask is taken as padded with that many all-False rows / columns in front (and at the end up to
+    whole tiles).  ``metadata`` is the MaskMetadata of that padded mask, ``padded_mask`` the padded mask itself
+    (the caller's mask when both offsets are 0 and no rounding up was needed)."""
+
+    BLOCK_Q: int
+    BLOCK_K: int
+    q_offset: int
+    k_offset: int
+    metadata: MaskMetadata
+    padded_mask: torch.Tensor
+    report: list
+
+
+def select_tiling(mask: torch.Tensor, candidates=DEFAULT_TILE_CANDIDATES, offsets: Sequence[Tuple[int, int]] = ((0, 0),),
+                  partial_cost: float = 1.25) -> Tiling:
+    """:func:`select_block_sizes` over tile sizes AND grid origins ("changing blocksizes / offsets to maximise the
+    number of totally masked-out blocks", README.md:64): every candidate (BLOCK_Q, BLOCK_K) is tried with every
+    ``(q_offset, k_offset)`` of ``offsets`` (0 <= offset < BLOCK; pairs that do not fit a candidate are skipped) on the
+    mask padded accordingly, priced like select_block_sizes does.  A mask whose structure has a period of the tile
+    size but starts off the grid (documents or windows that begin at row 32, say) loses its PARTIAL tiles at the
+    right origin.  Run the result with :func:`sparseattention_amd.sparse_attention_tiled`.  Reads counts back to the
+    host and copies the mask once per offset: call it once per mask."""
+    if mask.dim() != 4:
+        raise ValueError(f"mask must be [B,H,Sq,Sk] (got {tuple(mask.shape)})")
+    B, H, Sq, Sk = mask.shape
+    classify = compute_mask_kernel if mask.is_cuda else compute_mask_slow
+    distinct = mask[: 1 if mask.stride(0) == 0 else B, : 1 if mask.stride(1) == 0 else H]
+    best, report = None, []
+    for BQ, BK in candidates:
+        for qo, ko in offsets:
+            if not (0 <= qo < BQ and 0 <= ko < BK):
+                continue
+            pq, pk = -(Sq + qo) % BQ, -(Sk + ko) % BK
+            if (qo, ko, pq, pk) == (0, 0, 0, 0):
+                padded = mask
+            else:
+                padded = torch.nn.functional.pad(distinct, (ko, pk, qo, pq), value=False).expand(B, H, Sq + qo + pq, Sk + ko + pk)
+            md = classify(padded, BQ, BK)
+            full, part = int(md.unmasked_lens.sum()), int(md.masked_lens.sum())
+            cost = (full + partial_cost * part) * BQ * BK * entry_cost(BQ, BK)
+            report.append((BQ, BK, qo, ko, full, part, cost))
+            if best is None or cost < best[0]:
+                best = (cost, BQ, BK, qo, ko, md, padded)
+    if best is None:
+        raise ValueError("no candidate tile size / offset pair fits")
+    return Tiling(best[1], best[2], best[3], best[4], best[5], best[6], report)
+
+
 # ---- masks given by a formula -----------------------------------------------------------------------------------
 _TERM_BACK, _TERM_AHEAD, _TERM_Q_RANGE, _TERM_K_RANGE, _TERM_SAME_DOC = 1, 2, 4, 8, 16
 MAX_MASK_TERMS = 8

@@ -6,7 +6,7 @@ import math
 import torch
 
 from . import _native
-from .mask_utils import MaskMetadata, compute_mask_kernel, compute_mask_terms
+from .mask_utils import MaskMetadata, Tiling, compute_mask_kernel, compute_mask_terms
 
 _DTYPES = {torch.bfloat16: _native.SA_DTYPE_BF16, torch.float16: _native.SA_DTYPE_FP16}
 
@@ -230,6 +230,29 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
     if Dk != D:
         o = o[..., :D].contiguous()
     return (o, lse) if return_lse else o
+
+
+def sparse_attention_tiled(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, tiling: Tiling, *, return_lse: bool = False):
+    """:func:`sparse_attention` on the tile grid chosen by :func:`sparseattention_amd.select_tiling`: q, k, v get
+    ``q_offset`` / ``k_offset`` zero rows in front (and zero rows at the end up to whole tiles), which the padded mask
+    lets nothing attend to or from, and the rows of the result that belong to the caller's queries are returned.  With
+    both offsets 0 and sizes that are whole tiles this is sparse_attention itself; otherwise it costs a copy of q, k, v."""
+    Sq, Sk = q.shape[-2], k.shape[-2]
+    Pq, Pk = tiling.padded_mask.shape[-2:]
+    qo, ko = tiling.q_offset, tiling.k_offset
+    if not (qo + Sq <= Pq and ko + Sk <= Pk):
+        raise ValueError(f"tiling for a mask of {Pq - qo}x{Pk - ko} or smaller, got Sq={Sq}, Sk={Sk}")
+    pad = torch.nn.functional.pad
+    qp = q if (qo, Pq) == (0, Sq) else pad(q, (0, 0, qo, Pq - qo - Sq))
+    kp = k if (ko, Pk) == (0, Sk) else pad(k, (0, 0, ko, Pk - ko - Sk))
+    vp = v if (ko, Pk) == (0, Sk) else pad(v, (0, 0, ko, Pk - ko - Sk))
+    out = sparse_attention(qp, kp, vp, tiling.padded_mask, tiling.BLOCK_Q, tiling.BLOCK_K, tiling.metadata,
+                           return_lse=return_lse)
+    if (qo, Pq) == (0, Sq):
+        return out
+    if return_lse:
+        return out[0][:, :, qo:qo + Sq].contiguous(), out[1][:, :, qo:qo + Sq].contiguous()
+    return out[:, :, qo:qo + Sq].contiguous()
 
 
 def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor, BLOCK_K,

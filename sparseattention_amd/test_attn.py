@@ -38,20 +38,27 @@ def random_blocked_mask(B, Sq, Sk, BLOCK_Q, BLOCK_K, p, device="cuda"):
     return cells.to(torch.bool).to(device)
 
 
-def do_bench(fn, warmup=5, rep=20):
-    """Median time of fn() in ms, HIP events on the current stream."""
-    for _ in range(warmup):
-        fn()
-    times = []
-    for _ in range(rep):
-        start = torch.cuda.Event(enable_timing=True)
-        end = torch.cuda.Event(enable_timing=True)
+def do_bench(fn, warmup_ms=25.0, rep=20):
+    """Median time of fn() in ms: HIP events on the current stream around each of ``rep`` launches that follow each
+    other without a host synchronisation in between, after at least ``warmup_ms`` of untimed launches (as
+    triton.testing.do_bench warms up by time, test_attn.py:64-68: after the seconds of host work that make a mask the
+    device has dropped to a low power state and its first launches run several times slow)."""
+    import time
+
+    fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < warmup_ms:
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(rep)]
+    for start, end in pairs:
         start.record()
         fn()
         end.record()
-        end.synchronize()
-        times.append(start.elapsed_time(end))
-    times.sort()
+    torch.cuda.synchronize()
+    times = sorted(start.elapsed_time(end) for start, end in pairs)
     return times[len(times) // 2]
 
 

@@ -94,3 +94,52 @@ def test_pick_is_close_to_the_fastest_candidate_measured(gpu, kind):
     times = {c: timed(*c) for c in DEFAULT_TILE_CANDIDATES}
     fastest = min(times, key=times.get)
     assert times[(bq, bk)] <= 1.10 * times[fastest], f"picked {(bq, bk)}: {times[(bq, bk)]:.4f} ms, fastest {fastest}: {times[fastest]:.4f} ms; all {times}"
+
+
+def _shifted_blocks(S, block, shift):
+    """Block-diagonal mask whose blocks of `block` rows start `shift` rows after a multiple of `block`."""
+    i = torch.arange(S)
+    g = (i + block - shift) // block
+    return (g[:, None] == g[None, :])[None, None]
+
+
+def test_grid_origin_removes_partial_tiles_cpu():
+    from sparseattention_amd import select_tiling
+
+    mask = _shifted_blocks(1024, 128, 32)
+    t = select_tiling(mask, candidates=((128, 32), (128, 64)), offsets=((0, 0), (96, 0), (96, 32), (32, 32)))
+    assert (t.BLOCK_Q, t.q_offset) == (128, 96) and t.k_offset % 32 == 0
+    costs = {r[:4]: r for r in t.report}
+    # at the origin every block straddles two rows of tiles; with the grid moved by 96 rows none does
+    assert costs[(128, 32, 0, 0)][5] > 0 and costs[(128, 32, 96, 0)][4] > 0
+    assert costs[(128, 32, 96, 0)][6] < costs[(128, 32, 0, 0)][6]
+    assert t.padded_mask.shape[-2:] == (1024 + 96 + 32, 1024)
+    assert not t.padded_mask[0, 0, :96].any() and torch.equal(t.padded_mask[0, 0, 96:96 + 1024, :1024], mask[0, 0])
+    # offsets that do not fit a candidate are skipped, and (0, 0) alone is select_block_sizes
+    t0 = select_tiling(mask, candidates=((128, 32), (64, 64)))
+    bq, bk, md, _ = select_block_sizes(mask, candidates=((128, 32), (64, 64)))
+    assert (t0.BLOCK_Q, t0.BLOCK_K, t0.q_offset, t0.k_offset) == (bq, bk, 0, 0)
+    assert torch.equal(t0.metadata.unmasked_lens, md.unmasked_lens)
+
+
+@pytest.mark.gpu
+def test_forward_on_a_moved_grid(gpu):
+    import torch.nn.functional as F
+
+    from sparseattention_amd import select_tiling, sparse_attention, sparse_attention_tiled
+
+    B, H, S, D = 1, 2, 1024, 64
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=3, device=gpu)
+    mask = _shifted_blocks(S, 128, 32).to(gpu).expand(B, H, S, S)
+    t = select_tiling(mask, candidates=((128, 32), (128, 64)), offsets=((0, 0), (96, 0), (96, 32), (32, 32)))
+    assert (t.q_offset, t.k_offset % 32) == (96, 0)
+    o, lse = sparse_attention_tiled(q, k, v, t, return_lse=True)
+    want = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), attn_mask=mask)
+    assert o.shape == q.shape and (o.float() - want).abs().max() <= 2e-2
+    plain = sparse_attention(q, k, v, mask, 128, 32)
+    assert (o.float() - plain.float()).abs().max() <= 2e-2
+    s = torch.einsum("bhqd,bhkd->bhqk", q.float(), k.float()) / D ** 0.5
+    assert (lse - torch.logsumexp(s.masked_fill(~mask, float("-inf")), -1)).abs().max() <= 6e-3
+    # a tiling without offsets is sparse_attention itself
+    t0 = select_tiling(mask, candidates=((128, 32),))
+    assert torch.equal(sparse_attention_tiled(q, k, v, t0), plain)
