@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define SA_ABI_VERSION 12
+#define SA_ABI_VERSION 13
 
 enum sa_status {
     SA_OK = 0,
@@ -145,7 +145,9 @@ int sa_mask_classify_static(const uint8_t *mask, const int64_t mask_strides[4], 
  *
  * Supported: D in {64,128,256}; BQ in {32,64,128,256} (64 and 128 at D = 256, where a given schedule is not used);
  * BK a power of two >= 16.
- * ids[..., :len] must hold valid KV-tile indices (< Sk/BK): they address K and V directly.
+ * ids[..., :len] should hold valid KV-tile indices (< Sk/BK).  Counts are clamped to Sk/BK and an index outside
+ * [0, Sk/BK) is skipped, as the reference's masked loads would (sparse_attn_kernel.py:35,39,60); sa_validate_metadata
+ * tells whether that happened.
  */
 int sa_sparse_attention_fwd(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
                             const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
@@ -155,6 +157,21 @@ int sa_sparse_attention_fwd(const void *q, const int64_t q_strides[4], const voi
                             const int64_t part_ids_strides[4], const int32_t *part_lens,
                             const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int D, int BQ, int BK,
                             int dtype, float sm_scale_log2, void *stream);
+
+/*
+ * Check of caller-supplied lists before they are handed to a forward, decode or backward call, on the device and
+ * without a host synchronisation: the counterpart of the guard the reference puts on every K/V and mask load
+ * (kv_offset < SEQLEN_K, sparse_attn_kernel.py:35,39,60).  ORs into *flag (a device int32 the caller has set to 0):
+ *   1  a count is negative, or full_len + part_len exceeds Sk/BK for some Q tile
+ *   2  a FULL index inside its count is outside [0, Sk/BK)      4  the same for a PARTIAL index
+ * The caller reads the flag when it likes (with the results, say).  The attention kernels do not depend on it: they
+ * clamp counts to the row of tiles and skip (forward) or clamp (decode, backward) indices out of range, so lists that
+ * fail this check give wrong numbers, never an access outside the tensors.
+ */
+int sa_validate_metadata(const int32_t *full_ids, const int64_t full_ids_strides[4], const int32_t *full_lens,
+                         const int64_t full_lens_strides[3], const int32_t *part_ids, const int64_t part_ids_strides[4],
+                         const int32_t *part_lens, const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk,
+                         int BQ, int BK, int32_t *flag, void *stream);
 
 /*
  * Bytes of the buffer sa_mask_pack_partial fills: Sq*Sk/8 for every DISTINCT mask plane (room for every

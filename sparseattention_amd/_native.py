@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsparseattn_hip.so")
 
-SA_ABI_VERSION = 12
+SA_ABI_VERSION = 13
 SA_OK = 0
 SA_ERR_INVALID_ARGUMENT = -1
 SA_ERR_UNSUPPORTED = -2
@@ -30,6 +30,7 @@ EXPORTS = (
     "sa_mask_classify_workspace_bytes",
     "sa_mask_classify",
     "sa_mask_classify_static",
+    "sa_validate_metadata",
     "sa_sparse_attention_fwd",
     "sa_mask_pack_partial_bytes",
     "sa_mask_pack_partial",
@@ -84,6 +85,8 @@ def load() -> ctypes.CDLL:
     )
     lib.sa_mask_classify_static.restype = ctypes.c_int
     lib.sa_mask_classify_static.argtypes = [_vp, _i64p] + [ctypes.c_int] * 6 + [_vp, _i64p] * 4 + [_vp]
+    lib.sa_validate_metadata.restype = ctypes.c_int
+    lib.sa_validate_metadata.argtypes = [_vp, _i64p] * 4 + [ctypes.c_int] * 6 + [_vp, _vp]
     lib.sa_sparse_attention_fwd.restype = ctypes.c_int
     lib.sa_sparse_attention_fwd.argtypes = (
         [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [ctypes.c_int] * 8 + [ctypes.c_float, _vp]

@@ -54,6 +54,15 @@ struct ScheduleParams {
     int32_t *sched;
 };
 
+// Check of caller-supplied lists against the nK tiles a row of tiles has; *flag collects error bits (never cleared here).
+struct ValidateParams {
+    const int32_t *full_ids, *full_lens, *part_ids, *part_lens;
+    int64_t fis[4], fls[3], pis[4], pls[3];
+    int B, H, nQ, nK;
+    int32_t *flag;
+};
+hipError_t launch_validate(const ValidateParams &p, hipStream_t stream);
+
 hipError_t launch_classify(const ClassifyParams &p, bool wide, hipStream_t stream);
 hipError_t launch_schedule(const ScheduleParams &p, hipStream_t stream);
 hipError_t launch_compact(const CompactParams &p, hipStream_t stream);

@@ -182,7 +182,35 @@ __global__ __launch_bounds__(256) void pack_partial_kernel(const PackParams p) {
     }
 }
 
+// One wave per (b, h, Q tile) row of the lists: bit 0 of *flag when a count is negative or the two counts exceed nK,
+// bit 1 when a FULL index inside its count lies outside [0, nK), bit 2 the same for a PARTIAL index.
+__global__ __launch_bounds__(256) void validate_lists_kernel(const ValidateParams p) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= (int64_t)p.B * p.H * p.nQ) return;
+    const int qt = (int)(row % p.nQ);
+    const int h = (int)((row / p.nQ) % p.H);
+    const int b = (int)(row / ((int64_t)p.nQ * p.H));
+    const int nf = p.full_lens[b * p.fls[0] + h * p.fls[1] + qt * p.fls[2]];
+    const int np = p.part_lens[b * p.pls[0] + h * p.pls[1] + qt * p.pls[2]];
+    int bad = (nf < 0 || np < 0 || (int64_t)nf + np > p.nK) ? 1 : 0;
+    const int32_t *fid = p.full_ids + b * p.fis[0] + h * p.fis[1] + qt * p.fis[2];
+    const int32_t *pid = p.part_ids + b * p.pis[0] + h * p.pis[1] + qt * p.pis[2];
+    const int cf = nf < 0 ? 0 : (nf > p.nK ? p.nK : nf), cp = np < 0 ? 0 : (np > p.nK ? p.nK : np);  // slots that exist
+    for (int e = lane; e < cf; e += 64)
+        if ((unsigned)fid[(int64_t)e * p.fis[3]] >= (unsigned)p.nK) bad |= 2;
+    for (int e = lane; e < cp; e += 64)
+        if ((unsigned)pid[(int64_t)e * p.pis[3]] >= (unsigned)p.nK) bad |= 4;
+    if (bad) atomicOr(p.flag, bad);
+}
+
 }  // namespace
+
+hipError_t launch_validate(const ValidateParams &p, hipStream_t stream) {
+    const int64_t rows = (int64_t)p.B * p.H * p.nQ;
+    hipLaunchKernelGGL(validate_lists_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p);
+    return hipGetLastError();
+}
 
 hipError_t launch_pack(const PackParams &p, hipStream_t stream) {
     const int lanes = p.nK < 8 ? p.nK : 8;

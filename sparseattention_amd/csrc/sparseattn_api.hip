@@ -430,6 +430,39 @@ int sa_sparse_attention_fwd_lse(const void *q, const int64_t q_strides[4], const
                         lse, lse_strides, B, H, Sq, Sk, D, BQ, BK, dtype, sm_scale_log2, stream);
 }
 
+int sa_validate_metadata(const int32_t *full_ids, const int64_t full_ids_strides[4], const int32_t *full_lens,
+                         const int64_t full_lens_strides[3], const int32_t *part_ids, const int64_t part_ids_strides[4],
+                         const int32_t *part_lens, const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk,
+                         int BQ, int BK, int32_t *flag, void *stream) {
+    g_error[0] = 0;
+    if (!full_ids || !full_ids_strides || !full_lens || !full_lens_strides || !part_ids || !part_ids_strides ||
+        !part_lens || !part_lens_strides || !flag)
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_validate_metadata: null pointer argument");
+    if (const int rc = check_tiling(B, H, Sq, Sk, BQ, BK)) return rc;
+    if (!aligned(flag, 4)) return fail(SA_ERR_INVALID_ARGUMENT, "sa_validate_metadata: flag must be 4-byte aligned");
+    sa::ValidateParams vp{};
+    vp.full_ids = full_ids;
+    vp.full_lens = full_lens;
+    vp.part_ids = part_ids;
+    vp.part_lens = part_lens;
+    for (int i = 0; i < 4; i++) {
+        vp.fis[i] = full_ids_strides[i];
+        vp.pis[i] = part_ids_strides[i];
+    }
+    for (int i = 0; i < 3; i++) {
+        vp.fls[i] = full_lens_strides[i];
+        vp.pls[i] = part_lens_strides[i];
+    }
+    vp.B = B;
+    vp.H = H;
+    vp.nQ = Sq / BQ;
+    vp.nK = Sk / BK;
+    vp.flag = flag;
+    const hipError_t e = sa::launch_validate(vp, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_validate_metadata: launch failed: %s", hipGetErrorString(e));
+    return SA_OK;
+}
+
 size_t sa_fwd_schedule_bytes(int B, int H, int Sq, int Sk, int BQ, int BK, int mode) {
     return schedule_shape(B, H, Sq, Sk, BQ, BK, mode, nullptr, nullptr);
 }

@@ -250,3 +250,13 @@ def test_device_check_names_the_tensor():
     _same_device(ref, k=torch.empty(2, device="meta"), mask=None)
     with pytest.raises(ValueError, match="lse is on cpu"):
         _same_device(ref, k=torch.empty(2, device="meta"), lse=torch.empty(2))
+
+
+def test_validate_metadata_rejects_bad_arguments_on_the_host():
+    lib = _native.load()
+    args = lambda **kw: [kw.get("ids", FAKE), I4, FAKE, S3, FAKE, I4, FAKE, S3, 1, 1, kw.get("Sq", 64), 64, 32, 32,
+                         kw.get("flag", FAKE), None]  # noqa: E731
+    assert lib.sa_validate_metadata(*args(ids=None)) == _native.SA_ERR_INVALID_ARGUMENT
+    assert lib.sa_validate_metadata(*args(flag=None)) == _native.SA_ERR_INVALID_ARGUMENT
+    assert lib.sa_validate_metadata(*args(Sq=65)) == _native.SA_ERR_INVALID_ARGUMENT
+    assert lib.sa_validate_metadata(*args(flag=FAKE + 2)) == _native.SA_ERR_INVALID_ARGUMENT

@@ -226,3 +226,44 @@ def test_cpu_plumbing_workload_on_the_gpu(gpu, dtype):
         assert (o.float().cpu() - want).abs().max() <= TOL
     with pytest.raises(TypeError, match="float32"):
         sparse_attention(q32.to(gpu), k32.to(gpu), v32.to(gpu), me, 32, 32)
+
+
+def test_device_side_check_of_lists(gpu):
+    # sa_validate_metadata: error bits in a device int, no host synchronisation on the way
+    lib = _native.load()
+    S_ = _native.strides
+    B, H, S, BQ, BK = 2, 3, 1024, 128, 32
+    nK = S // BK
+    mask = W.random_block_mask(S, 128, 0.5, seed=9, device=gpu, batch=B).expand(B, H, S, S)
+    md = compute_mask_kernel(mask, BQ, BK, pack_partial=False)
+
+    def check(md_):
+        flag = torch.zeros(1, dtype=torch.int32, device=gpu)
+        rc = lib.sa_validate_metadata(
+            md_.unmasked_kv_ids.data_ptr(), S_(md_.unmasked_kv_ids.stride()), md_.unmasked_lens.data_ptr(), S_(md_.unmasked_lens.stride()),
+            md_.masked_kv_ids.data_ptr(), S_(md_.masked_kv_ids.stride()), md_.masked_lens.data_ptr(), S_(md_.masked_lens.stride()),
+            B, H, S, S, BQ, BK, flag.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        _native.check(rc)
+        return int(flag.item())
+
+    assert check(md) == 0  # broadcast (stride-0) views as compute_mask_kernel returns them
+    assert check(compute_mask_slow(mask, BQ, BK)) == 0  # -1 in the unused slots does not count
+    own = lambda: MaskMetadata(md.unmasked_kv_ids.contiguous().clone(), md.unmasked_lens.contiguous().clone(),  # noqa: E731
+                               md.masked_kv_ids.contiguous().clone(), md.masked_lens.contiguous().clone())
+    bad = own()
+    bad.unmasked_lens[1, 2, 3] = nK + 1
+    assert check(bad) & 1
+    bad = own()
+    bad.masked_lens[0, 0, 0] = -2
+    assert check(bad) == 1
+    bad = own()
+    b, h, t = (int(x) for x in torch.nonzero(bad.unmasked_lens > 0)[-1])  # some Q tile that has a FULL tile
+    bad.unmasked_kv_ids[b, h, t, 0] = nK
+    assert check(bad) == 2
+    bad = own()
+    b, h, t = (int(x) for x in torch.nonzero(bad.masked_lens > 0)[0])
+    bad.masked_kv_ids[b, h, t, int(bad.masked_lens[b, h, t]) - 1] = -1
+    assert check(bad) == 4
+    # and the Python check agrees
+    with pytest.raises(ValueError):
+        validate_metadata(bad, S, BK)
