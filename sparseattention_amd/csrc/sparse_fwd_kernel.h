@@ -1028,6 +1028,12 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
             static_for<EPC>([&](auto j_c) { raw0[decltype(j_c)::value] = early_entry(j_c); });
             entries_use(0, raw0, col, valid, part);
             stage_chunk(0, col);
+            // (and its mask words, when it has a PARTIAL or absent entry: where every tile is PARTIAL they were the
+            // last thing a Q tile waited for before its loop)
+            sp[0] = part != 0u || valid != ALL;
+            vl[0] = valid;
+            pt[0] = part;
+            if (sp[0]) load_mask(0, col, mk[0], MaskSrc{mrow, prow, F, NE});
             const bool mine = list_in_lds && tid < list_cnt;
             int first_slots = 0;
             if (mine) first_slots = tagged_entry(tid);
@@ -1043,11 +1049,11 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
         } else {
             chunk_entries(0, col, valid, part);
             stage_chunk(0, col);
+            sp[0] = part != 0u || valid != ALL;
+            vl[0] = valid;
+            pt[0] = part;
+            if (sp[0]) load_mask(0, col, mk[0], MaskSrc{mrow, prow, F, NE});
         }
-        sp[0] = part != 0u || valid != ALL;
-        vl[0] = valid;
-        pt[0] = part;
-        if (sp[0]) load_mask(0, col, mk[0], MaskSrc{mrow, prow, F, NE});
         chunk_entries(1 < T ? 1 : 0, coln, valid, part);
         sp[1] = 1 < T && (part != 0u || valid != ALL);
         vl[1] = valid;
