@@ -41,23 +41,39 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak, TFLOP/s
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E peak, GB/s
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this script and scaled by
-# the readings of a 1 GiB device copy in the same run (--calibrate-copy).  The summaries with the commands
-# are profiles/sparse_fwd_kernel_causal_B8H32S4096D128.txt and profiles/mask_classify_kernels_mask_32768x32768.txt.
-TRAFFIC_FWD_CAUSAL_BYTES = 1.1708e9      # 860.6 MiB read + 256.0 MiB written
-TRAFFIC_CLASSIFY_1GIB_BYTES = 1.0744e9   # 1,048,622 + 327 KiB read, 256 + 45.5 KiB written
-# decode workloads (profiles/sparse_decode_kernel_B8H32Sk32768D128.txt), both kernels
-TRAFFIC_DECODE_BYTES = (4.2959e9, 1.6225e9)
-# backward of the headline workload (profiles/sparse_bwd_kernel_causal_B8H32S4096D128.txt), three passes + prepare:
-# 4242 MiB read + 776 MiB written
-TRAFFIC_BWD_CAUSAL_BYTES = 5.262e9
+# the readings of a 1 GiB device copy in the same run (--calibrate-copy: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000
+# KiB).  The summaries with the commands are the files of TRAFFIC_SOURCE.
+TRAFFIC_FWD_CAUSAL_BYTES = 1.1111e9      # 803.6 MiB read + 256.0 MiB written
+TRAFFIC_CLASSIFY_1GIB_BYTES = 1.0744e9   # 1,048,628 + 327 KiB read, 256 + 45.5 KiB written
+# decode workloads, both kernels
+TRAFFIC_DECODE_BYTES = (4.2963e9, 1.6227e9)
+# backward of the headline workload, three passes + prepare: 4167.8 MiB read + 776 MiB written
+TRAFFIC_BWD_CAUSAL_BYTES = 5.184e9
 
-# where the constants above come from (refreshed whenever a kernel changes: same commands as in the files)
+# where the constants above come from
 TRAFFIC_SOURCE = {
     "forward": "profiles/sparse_fwd_kernel_causal_B8H32S4096D128.txt section 2",
     "mask_classify": "profiles/mask_classify_kernels_mask_32768x32768.txt section 2",
     "decode": "profiles/sparse_decode_kernel_B8H32Sk32768D128.txt",
     "backward": "profiles/sparse_bwd_kernel_causal_B8H32S4096D128.txt",
 }
+# The counters were read with the kernels built from sources of this digest (kernel_sources_sha16 below); the line
+# carries both digests, so a reader sees whether the traffic figures belong to the kernels that were timed.
+TRAFFIC_KERNEL_SOURCES_SHA16 = "8275a056bd0c7a4b"
+
+
+def kernel_sources_sha16():
+    """First 16 hex digits of the SHA-256 over the kernel sources (names and contents, in name order)."""
+    import glob
+    import hashlib
+
+    h = hashlib.sha256()
+    for f in sorted(glob.glob(os.path.join(ROOT, "sparseattention_amd", "csrc", "*"))):
+        h.update(os.path.basename(f).encode())
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
 
 SETTLE_LAUNCHES = 30
 SETTLE_MS = 40.0
@@ -461,6 +477,8 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_FWD_CAUSAL_BYTES,
                      "traffic_source": TRAFFIC_SOURCE["forward"],
+                     "traffic_kernel_sources_sha16": TRAFFIC_KERNEL_SOURCES_SHA16,
+                     "kernel_sources_sha16": kernel_sources_sha16(),
                      "kernel": "sparse_fwd_kernel", "kernel_ms": head["kernel_ms"],
                      "flop_per_launch": head["_executed_flop"]},
     }
