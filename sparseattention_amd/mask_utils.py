@@ -6,7 +6,7 @@ Mirrors the interface of the reference's ``sparseattention/mask_utils.py``:
 from __future__ import annotations
 
 import ctypes
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Optional, Sequence, Tuple
 
 import torch
@@ -34,6 +34,11 @@ class MaskMetadata:
     row: the count; then ``((b << 16) | h, qt, unmasked_len, masked_len)`` per tile), made by
     ``compute_mask_kernel(..., schedule="pairs" | "persistent")``.  It depends on the counts, on B and H and, for
     "persistent", on the device; without it the forward launches one workgroup per Q tile.
+
+    Two book-keeping fields follow, neither compared nor shown: ``_validated_for`` = the ``(Sk, BLOCK_K)`` these lists
+    have been checked against (set by the functions of this module, whose lists fit by construction, and by
+    ``sparse_attention`` after it has checked a caller-built object once), and ``_retiled`` = the lists of the same
+    mask at tile sizes the kernels have, kept by ``sparse_attention`` when it was asked for sizes they do not have.
     """
 
     unmasked_kv_ids: torch.Tensor
@@ -43,6 +48,8 @@ class MaskMetadata:
     packed_masks: Optional[torch.Tensor] = None
     schedule: Optional[torch.Tensor] = None
     schedule_mode: int = 0
+    _validated_for: Optional[Tuple[int, int]] = field(default=None, repr=False, compare=False)
+    _retiled: Optional[tuple] = field(default=None, repr=False, compare=False)
 
 
 def _check_mask(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int):

@@ -78,7 +78,7 @@ def _checked_metadata(md: MaskMetadata, Sk: int, BLOCK_K: int) -> None:
     validate_metadata(md, Sk, BLOCK_K)
     try:
         md._validated_for = key
-    except AttributeError:  # a carrier that takes no new attributes is simply checked again next time
+    except AttributeError:  # the reference's own dataclass, say: a carrier without the field is checked every time
         pass
 
 
