@@ -432,6 +432,21 @@ def cpu_baselines():
         "ms_full_workload": round(dt * 1e3 * B * H / hs, 1),
         "host_cpu_count": os.cpu_count(),
     }
+    del q, k, v
+    # (c) preprocessing on the CPU: the vectorised restatement of the reference's classification loop
+    # (compute_mask_slow, mask_utils.py:14-44) on the first 4096 rows of the composed S = 32768 mask
+    from sparseattention_amd import compute_mask_slow
+
+    rows = 4096
+    big = W.composed_mask(32768)[:rows][None, None]
+    t0 = time.perf_counter()
+    compute_mask_slow(big, BQ, BK)
+    dt = time.perf_counter() - t0
+    out["mask_classify_cpu_baseline"] = {
+        "value": round(big.numel() / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"compute_mask_slow (plain torch on CPU tensors) on the first {rows} of the 32768 rows of the composed "
+                  f"mask, 128 MiB of the 1 GiB, tiles {BQ}x{BK}: {dt:.2f} s, mask bytes per second",
+    }
     return out
 
 
