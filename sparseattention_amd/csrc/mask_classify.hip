@@ -142,8 +142,10 @@ __global__ __launch_bounds__(256) void compact_kernel(const CompactParams p) {
     }
 }
 
-// grid (slot lanes, nQ, distinct planes), 256 threads.  Workgroup x takes the PARTIAL slots x, x + gridDim.x, ...
-// of its Q tile; a thread makes one output byte at a time from 8 neighbouring mask entries of one row.
+// grid (slot lanes, nQ, distinct planes), 256 threads.  Workgroup x takes a run of consecutive PARTIAL slots of its Q
+// tile, at least four: neighbouring tiles share the 128-byte lines of the mask rows (four tiles of 32 keys per line),
+// and the workgroups of one Q tile run on different XCDs, each with an L2 of its own.  A thread makes one output
+// byte at a time from 8 neighbouring mask entries of one row.
 __global__ __launch_bounds__(256) void pack_partial_kernel(const PackParams p) {
     const int qt = blockIdx.y;
     const int plane = blockIdx.z;
@@ -154,7 +156,9 @@ __global__ __launch_bounds__(256) void pack_partial_kernel(const PackParams p) {
     const int tile_bytes = p.BQ * bpr;
     const uint8_t *rows = p.mask + (int64_t)ub * p.sb + (int64_t)uh * p.sh + (int64_t)qt * p.BQ * p.sq;
     uint8_t *out_q = p.packed + (int64_t)ub * p.ob + (int64_t)uh * p.oh + (int64_t)qt * p.nK * tile_bytes;
-    for (int slot = blockIdx.x; slot < len; slot += gridDim.x) {
+    const int per = max(4, (len + (int)gridDim.x - 1) / (int)gridDim.x);
+    const int slot_end = min(len, ((int)blockIdx.x + 1) * per);
+    for (int slot = blockIdx.x * per; slot < slot_end; slot++) {
         const int64_t col0 = (int64_t)ids[(int64_t)slot * p.pis[3]] * p.BK;
         uint8_t *out = out_q + (int64_t)slot * tile_bytes;
         for (int o = threadIdx.x; o < tile_bytes; o += 256) {
