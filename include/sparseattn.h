@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define SA_ABI_VERSION 13
+#define SA_ABI_VERSION 14
 
 enum sa_status {
     SA_OK = 0,
@@ -50,7 +50,8 @@ enum sa_status {
 
 enum sa_dtype {
     SA_DTYPE_BF16 = 0,
-    SA_DTYPE_FP16 = 1
+    SA_DTYPE_FP16 = 1,
+    SA_DTYPE_FP32 = 2 /* the forward entry points only (sa_sparse_attention_fwd, _fwd_ex, _fwd_lse) */
 };
 
 /* Conditions of one term of a mask given by a formula (sa_mask_classify_terms). */
@@ -145,6 +146,10 @@ int sa_mask_classify_static(const uint8_t *mask, const int64_t mask_strides[4], 
  *
  * Supported: D in {64,128,256}; BQ in {32,64,128,256} (64 and 128 at D = 256, where a given schedule is not used);
  * BK a power of two >= 16.
+ * dtype SA_DTYPE_FP32 (the reference's kernel takes whatever element type its inputs have,
+ * sparse_attn_kernel.py:98-101, :145): q, k, v, o are float, strides multiples of 4 elements; a plain kernel on the
+ * vector units that keeps everything in float32 (P is not rounded), for checks against fp32 references, not for speed;
+ * any BQ from 1 to 256 (to 128 at D = 256) and any BK that divide Sq and Sk; a schedule is not used.
  * ids[..., :len] should hold valid KV-tile indices (< Sk/BK).  Counts are clamped to Sk/BK and an index outside
  * [0, Sk/BK) is skipped, as the reference's masked loads would (sparse_attn_kernel.py:35,39,60); sa_validate_metadata
  * tells whether that happened.

@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsparseattn_hip.so")
 
-SA_ABI_VERSION = 13
+SA_ABI_VERSION = 14
 SA_OK = 0
 SA_ERR_INVALID_ARGUMENT = -1
 SA_ERR_UNSUPPORTED = -2
@@ -19,6 +19,7 @@ SA_ERR_HIP = -4
 
 SA_DTYPE_BF16 = 0
 SA_DTYPE_FP16 = 1
+SA_DTYPE_FP32 = 2  # forward only
 
 SA_SCHEDULE_PERSISTENT = 0
 SA_SCHEDULE_PAIRS = 1

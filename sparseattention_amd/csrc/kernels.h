@@ -128,6 +128,9 @@ struct FwdParams {
 
 // dtype: 0 bf16, 1 fp16.  Returns hipErrorInvalidValue when no instantiation matches (D, BQ).
 hipError_t launch_fwd(const FwdParams &p, int dtype, int D, int BQ, hipStream_t stream);
+// float32 q, k, v, o (the pointers of FwdParams then address floats; strides stay in elements): any BQ from 1 to 256
+// (to 128 at D = 256), any BK; reads the packed tiles when given, else the mask; no schedules.
+hipError_t launch_fwd_f32(const FwdParams &p, int D, int BQ, hipStream_t stream);
 
 // Few query rows against a long K/V (decode): one Q tile of Sq <= 32 rows per (b, h), its list of KV tiles split
 // over `nsplit` workgroups whose partial results a second kernel merges.

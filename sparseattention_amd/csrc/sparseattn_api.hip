@@ -259,30 +259,40 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
     if (D <= 0) return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd: D must be positive (got %d)", D);
     if (!(sm_scale_log2 > 0.f) || !(sm_scale_log2 < 3.0e38f))
         return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd: sm_scale_log2 must be positive and finite");
-    if (dtype != SA_DTYPE_BF16 && dtype != SA_DTYPE_FP16)
-        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: dtype code %d (supported: 0 = bf16, 1 = fp16)", dtype);
+    const bool f32 = dtype == SA_DTYPE_FP32;  // the plain float32 kernel: any BLOCK_Q up to 256, any BLOCK_K
+    if (dtype != SA_DTYPE_BF16 && dtype != SA_DTYPE_FP16 && !f32)
+        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: dtype code %d (supported: 0 = bf16, 1 = fp16, 2 = fp32)", dtype);
     if (D != 64 && D != 128 && D != 256)
         return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: head dim %d (supported: 64, 128, 256)", D);
-    if (BQ != 32 && BQ != 64 && BQ != 128 && BQ != 256)
-        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: BLOCK_Q %d (supported: 32, 64, 128, 256)", BQ);
-    if (D == 256 && BQ != 64 && BQ != 128)
-        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: BLOCK_Q %d at head dim 256 (supported there: 64, 128)", BQ);
-    const int lbk = log2_exact(BK);
-    if (lbk < 4) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: BLOCK_K %d (supported: powers of two >= 16)", BK);
+    int lbk = 0;
+    if (f32) {
+        if (use_packed && BK % 8 != 0)
+            return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd: packed tiles need BLOCK_K to be a multiple of 8 (got %d)", BK);
+        if (BQ > (D > 128 ? 128 : 256))
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: BLOCK_Q %d in float32 (supported: 1 to 256, to 128 at head dim 256)", BQ);
+    } else {
+        if (BQ != 32 && BQ != 64 && BQ != 128 && BQ != 256)
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: BLOCK_Q %d (supported: 32, 64, 128, 256)", BQ);
+        if (D == 256 && BQ != 64 && BQ != 128)
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: BLOCK_Q %d at head dim 256 (supported there: 64, 128)", BQ);
+        lbk = log2_exact(BK);
+        if (lbk < 4) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: BLOCK_K %d (supported: powers of two >= 16)", BK);
+    }
     const int64_t *st[4] = {q_strides, k_strides, v_strides, o_strides};
     const void *ptr[4] = {q, k, v, o};
     const char *name[4] = {"q", "k", "v", "o"};
+    const int per16 = f32 ? 4 : 8;  // elements in 16 bytes
     for (int t = 0; t < 4; t++) {
         if (st[t][3] != 1 && D != 1)
             return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: %s must be contiguous in its last dimension (stride %lld)", name[t], (long long)st[t][3]);
-        if (!aligned(ptr[t], 16) || st[t][0] % 8 || st[t][1] % 8 || st[t][2] % 8)
-            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: %s needs a 16-byte aligned base and strides that are multiples of 8 elements", name[t]);
+        if (!aligned(ptr[t], 16) || st[t][0] % per16 || st[t][1] % per16 || st[t][2] % per16)
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: %s needs a 16-byte aligned base and strides that are multiples of %d elements", name[t], per16);
     }
     if (o_strides[2] == 0 || (B > 1 && o_strides[0] == 0) || (H > 1 && o_strides[1] == 0))
         return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd: o must not alias itself (zero stride)");
     if (Sk >= (1 << 30)) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: Sk %d (supported: below 2^30)", Sk);
     // (the kernels form row offsets of K and V from 32-bit factors)
-    if (k_strides[2] < 0 || v_strides[2] < 0 || k_strides[2] >= (1 << 24) || v_strides[2] >= (1 << 24))
+    if (!f32 && (k_strides[2] < 0 || v_strides[2] < 0 || k_strides[2] >= (1 << 24) || v_strides[2] >= (1 << 24)))
         return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: row strides of k and v must lie in [0, 2^24) elements (%lld, %lld)",
                     (long long)k_strides[2], (long long)v_strides[2]);
     if ((int64_t)B * H * (Sq / BQ) > 0x7fffffffLL)
@@ -316,7 +326,7 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
     fp.pks[1] = use_packed ? packed_strides[1] : 0;
     fp.nK = Sk / BK;
     fp.sched = nullptr;
-    if (schedule && D <= 128) {  // head dim 256 has no scheduled kernels; the order of Q tiles does not change results
+    if (schedule && D <= 128 && !f32) {  // head dim 256 and float32 have no scheduled kernels; the order of Q tiles does not change results
         int G = 0, R = 0;
         const size_t want = schedule_shape(B, H, Sq, Sk, BQ, BK, schedule_mode, &G, &R);
         if (want != 0 && want == schedule_bytes) {
@@ -347,7 +357,8 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
         fp.lse = lse;
         for (int i = 0; i < 3; i++) fp.lses[i] = lse_strides[i];
     }
-    const hipError_t e = sa::launch_fwd(fp, dtype, D, BQ, static_cast<hipStream_t>(stream));
+    const hipError_t e = f32 ? sa::launch_fwd_f32(fp, D, BQ, static_cast<hipStream_t>(stream))
+                             : sa::launch_fwd(fp, dtype, D, BQ, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_fwd: launch failed: %s", hipGetErrorString(e));
     return SA_OK;
 }

@@ -9,11 +9,14 @@ from . import _native
 from .mask_utils import MaskMetadata, Tiling, compute_mask_kernel, compute_mask_terms
 
 _DTYPES = {torch.bfloat16: _native.SA_DTYPE_BF16, torch.float16: _native.SA_DTYPE_FP16}
+# the forward also takes float32 (a plain kernel on the vector units, for checks against fp32 references)
+_FWD_DTYPES = {**_DTYPES, torch.float32: _native.SA_DTYPE_FP32}
 
 
 def _kernel_ready(t: torch.Tensor) -> torch.Tensor:
     """The kernels want a unit stride in D, 16-byte aligned rows; copy only when that does not hold."""
-    ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in t.stride()[:-1])
+    per16 = 16 // t.element_size()
+    ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % per16 == 0 for s in t.stride()[:-1])
     return t if ok else t.contiguous()
 
 
@@ -112,7 +115,8 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
     """softmax(q kᵀ / sqrt(D) + (mask ? 0 : -inf)) v, skipping KV tiles the mask empties.
 
     Signature and meaning follow sparse_attn_kernel.py:149-185: ``q`` [B,H,Sq,D], ``k``/``v``
-    [B,H,Sk,D] (bf16 or fp16, on a ROCm GPU), ``mask`` bool broadcastable to [B,H,Sq,Sk] with
+    [B,H,Sk,D] (bf16 or fp16 on the tuned kernels; float32 on a plain kernel that computes in float32 throughout; on a
+    ROCm GPU), ``mask`` bool broadcastable to [B,H,Sq,Sk] with
     True = attend, tile sizes ``BLOCK_Q`` x ``BLOCK_K``, and optionally the metadata from
     :func:`compute_mask_kernel` so that preprocessing is paid once for many calls.
     Returns ``o`` with q's shape, dtype and strides; with ``return_lse=True`` (not in the reference, which drops
@@ -130,15 +134,18 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
     if not q.is_cuda:
         raise RuntimeError("sparse_attention needs q, k, v on a ROCm GPU; there is no CPU path")
     _same_device(q, k=k, v=v, mask=mask)
-    if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
-        raise TypeError(f"q, k, v must share dtype bfloat16 or float16 (got {q.dtype}, {k.dtype}, {v.dtype}); "
-                        "float32 inputs, which the reference's kernel accepts, have no kernel here: cast them")
+    if q.dtype not in _FWD_DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise TypeError(f"q, k, v must share dtype bfloat16, float16 or float32 (got {q.dtype}, {k.dtype}, {v.dtype})")
+    f32 = q.dtype == torch.float32
     if mask is None and getattr(mask_metadata, "packed_masks", None) is None:
         raise ValueError("sparse_attention without a mask tensor needs mask_metadata with packed_masks")
     if mask is not None:
         mask = mask.expand(B, H, Sq, Sk)
     BLOCK_Q, BLOCK_K = int(BLOCK_Q), int(BLOCK_K)
-    tiles = kernel_tiles(Sq, Sk, D, BLOCK_Q, BLOCK_K)
+    if f32 and 1 <= BLOCK_Q <= (256 if D <= 128 else 128) and BLOCK_K >= 1 and Sq % BLOCK_Q == 0 and Sk % BLOCK_K == 0:
+        tiles = (BLOCK_Q, BLOCK_K)  # the float32 kernel tiles by any sizes up to 256 query rows (128 at head dims above 128)
+    else:
+        tiles = kernel_tiles(Sq, Sk, D, BLOCK_Q, BLOCK_K)
     row_multiple = 32 if D <= 128 else 64  # the smallest Q tile the kernels have
     if tiles is None and mask is not None and Sq % row_multiple and Sq % BLOCK_Q == 0 and Sk % BLOCK_K == 0:
         # A row count that no Q tile of the kernels divides (48, 80, ...; fewer than 32 rows at a head dim the few-rows
@@ -169,7 +176,7 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
         BLOCK_Q, BLOCK_K = tiles
         mask_metadata = again[1]
 
-    if Sq == BLOCK_Q and Sq < 32 and BLOCK_K >= 32:
+    if Sq == BLOCK_Q and Sq < 32 and BLOCK_K >= 32 and not f32:
         # one Q tile of fewer rows than the forward kernels tile by: the split-KV kernels.  They read the bool mask and
         # use neither packed tiles nor a schedule, so metadata that carries those (compute_mask_kernel's default) runs too.
         if mask is None:
@@ -212,7 +219,7 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
                   mask.data_ptr() if mask is not None else None, S(mask.stride()) if mask is not None else None,
                   fid.data_ptr(), S(fid.stride()), fl.data_ptr(), S(fl.stride()),
                   pid.data_ptr(), S(pid.stride()), pl.data_ptr(), S(pl.stride()))
-        tail = (B, H, Sq, Sk, Dk, int(BLOCK_Q), int(BLOCK_K), _DTYPES[q.dtype], sm_scale,
+        tail = (B, H, Sq, Sk, Dk, int(BLOCK_Q), int(BLOCK_K), _FWD_DTYPES[q.dtype], sm_scale,
                 torch.cuda.current_stream(q.device).cuda_stream)
         sched = getattr(mask_metadata, "schedule", None)
         lse = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device) if return_lse else None

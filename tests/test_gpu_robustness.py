@@ -224,8 +224,6 @@ def test_cpu_plumbing_workload_on_the_gpu(gpu, dtype):
         assert_metadata_equal(md, oracle.classify(mask.numpy()[None, None].repeat(H, 1), BQ, BK), f"{BQ}x{BK}")
         o = sparse_attention(q, k, v, me, BQ, BK, md)
         assert (o.float().cpu() - want).abs().max() <= TOL
-    with pytest.raises(TypeError, match="float32"):
-        sparse_attention(q32.to(gpu), k32.to(gpu), v32.to(gpu), me, 32, 32)
 
 
 def test_device_side_check_of_lists(gpu):
