@@ -94,6 +94,12 @@ def test_forward_rejects_bad_arguments():
     assert fwd(BK=8) == _native.SA_ERR_UNSUPPORTED and "BLOCK_K" in last_error()
     assert fwd(BK=4, Sk=252, Sq=256) == _native.SA_ERR_UNSUPPORTED
     assert fwd(dtype=7) == _native.SA_ERR_UNSUPPORTED and "dtype" in last_error()
+    # float32 (dtype 2): any BLOCK_Q up to 256 (128 at head dim 256), strides in multiples of four elements
+    f32 = _native.SA_DTYPE_FP32
+    assert fwd(dtype=f32, BQ=512, Sq=512) == _native.SA_ERR_UNSUPPORTED and "float32" in last_error()
+    assert fwd(dtype=f32, D=256, BQ=256) == _native.SA_ERR_UNSUPPORTED and "float32" in last_error()
+    assert fwd(dtype=f32, D=96) == _native.SA_ERR_UNSUPPORTED and "head dim" in last_error()
+    assert fwd(dtype=f32, qs=_native.strides((256 * 128, 256 * 128, 130, 1))) == _native.SA_ERR_UNSUPPORTED
     assert fwd(q=FAKE + 2) == _native.SA_ERR_UNSUPPORTED and "aligned" in last_error()
     assert fwd(qs=_native.strides((256 * 128, 256 * 128, 128, 2))) == _native.SA_ERR_UNSUPPORTED
     assert fwd(qs=_native.strides((256 * 128, 256 * 128, 132, 1))) == _native.SA_ERR_UNSUPPORTED
