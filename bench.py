@@ -43,12 +43,12 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E peak, GB/s
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this script and scaled by
 # the readings of a 1 GiB device copy in the same run (--calibrate-copy: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000
 # KiB).  The summaries with the commands are the files of TRAFFIC_SOURCE.
-TRAFFIC_FWD_CAUSAL_BYTES = 1.1304e9      # 821.9 MiB read + 256.0 MiB written (804 - 822 MiB read from run to run)
+TRAFFIC_FWD_CAUSAL_BYTES = 1.1748e9      # 864.3 MiB read + 256.0 MiB written (804 - 864 MiB read from box to box)
 TRAFFIC_CLASSIFY_1GIB_BYTES = 1.0744e9   # 1,048,628 + 327 KiB read, 256 + 45.5 KiB written
 # decode workloads, both kernels
 TRAFFIC_DECODE_BYTES = (4.2963e9, 1.6227e9)
-# backward of the headline workload, three passes + prepare: 4311.2 MiB read + 776 MiB written (4168 - 4311 MiB read)
-TRAFFIC_BWD_CAUSAL_BYTES = 5.334e9
+# backward of the headline workload, three passes + prepare: 4253.6 MiB read + 776 MiB written (4168 - 4311 MiB read)
+TRAFFIC_BWD_CAUSAL_BYTES = 5.274e9
 
 # where the constants above come from
 TRAFFIC_SOURCE = {
@@ -59,7 +59,7 @@ TRAFFIC_SOURCE = {
 }
 # The counters were read with the kernels built from sources of this digest (kernel_sources_sha16 below); the line
 # carries both digests, so a reader sees whether the traffic figures belong to the kernels that were timed.
-TRAFFIC_KERNEL_SOURCES_SHA16 = "99b8febc0c402676"
+TRAFFIC_KERNEL_SOURCES_SHA16 = "f33b103d9f0f16d7"
 
 
 def kernel_sources_sha16():

@@ -170,7 +170,9 @@ def test_wrapper_errors(gpu):
     q = torch.zeros(1, 1, 128, 128, device=gpu)
     m = torch.ones(128, 128, dtype=torch.bool, device=gpu)
     with pytest.raises(TypeError):
-        sparse_attention(q, q, q, m, 128, 32)  # fp32 has no kernel
+        sparse_attention(q.double(), q.double(), q.double(), m, 128, 32)  # bf16, fp16 and fp32 only
+    with pytest.raises(TypeError):
+        sparse_attention(q, q.bfloat16(), q, m, 128, 32)  # one element type for all three
     qb = torch.zeros(1, 1, 128, 512, dtype=torch.bfloat16, device=gpu)
     with pytest.raises(_native.SparseAttnError, match="head dim"):
         sparse_attention(qb, qb, qb, m, 128, 32)
