@@ -25,6 +25,9 @@ the reference also excludes preprocessing from the forward time and reports it s
   tile_selection   every candidate tile size of select_block_sizes timed on four masks, next to what it picked
   cpu_baseline     torch's masked SDPA on CPU tensors of the whole workload: the reference's own check path
                    (test_attn.py:40) on the host cores; cpu_oracle_baseline: the C oracle (a port) on the same workload
+                   mask_classify_cpu_baseline: compute_mask_slow (plain torch) on CPU tensors of a slab of the 1 GiB mask
+  roofline.traffic  HBM bytes per launch from rocprofv3 counter runs (a constant here: traffic_source names the summary,
+                   traffic_kernel_sources_sha16 the kernel sources it was read with, kernel_sources_sha16 the ones timed)
 """
 import argparse
 import gc
