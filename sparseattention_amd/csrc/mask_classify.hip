@@ -146,11 +146,14 @@ __global__ __launch_bounds__(256) void compact_kernel(const CompactParams p) {
 // tile, at least four: neighbouring tiles share the 128-byte lines of the mask rows (four tiles of 32 keys per line),
 // and the workgroups of one Q tile run on different XCDs, each with an L2 of its own.  A thread makes one output
 // byte at a time from 8 neighbouring mask entries of one row.
+// The lists may be a caller's own: the count is clamped to the nK slots a Q tile has in `packed`, and a slot whose
+// index lies outside [0, nK) is left untouched, so neither the reads of the mask nor the writes of `packed` leave
+// their tensors whatever the lists hold.
 __global__ __launch_bounds__(256) void pack_partial_kernel(const PackParams p) {
     const int qt = blockIdx.y;
     const int plane = blockIdx.z;
     const int ub = plane / p.uH, uh = plane - ub * p.uH;
-    const int len = p.part_lens[ub * p.pls[0] + uh * p.pls[1] + qt * p.pls[2]];
+    const int len = min(max(p.part_lens[ub * p.pls[0] + uh * p.pls[1] + qt * p.pls[2]], 0), p.nK);
     const int32_t *ids = p.part_ids + ub * p.pis[0] + uh * p.pis[1] + qt * p.pis[2];
     const int bpr = p.BK >> 3;                 // output bytes per tile row
     const int tile_bytes = p.BQ * bpr;
@@ -159,7 +162,9 @@ __global__ __launch_bounds__(256) void pack_partial_kernel(const PackParams p) {
     const int per = max(4, (len + (int)gridDim.x - 1) / (int)gridDim.x);
     const int slot_end = min(len, ((int)blockIdx.x + 1) * per);
     for (int slot = blockIdx.x * per; slot < slot_end; slot++) {
-        const int64_t col0 = (int64_t)ids[(int64_t)slot * p.pis[3]] * p.BK;
+        const int id = ids[(int64_t)slot * p.pis[3]];
+        if ((unsigned)id >= (unsigned)p.nK) continue;  // (uniform over the workgroup)
+        const int64_t col0 = (int64_t)id * p.BK;
         uint8_t *out = out_q + (int64_t)slot * tile_bytes;
         for (int o = threadIdx.x; o < tile_bytes; o += 256) {
             const int r = o / bpr, cb = o - r * bpr;

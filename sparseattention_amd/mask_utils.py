@@ -35,9 +35,11 @@ class MaskMetadata:
     ``compute_mask_kernel(..., schedule="pairs" | "persistent")``.  It depends on the counts, on B and H and, for
     "persistent", on the device; without it the forward launches one workgroup per Q tile.
 
-    Two book-keeping fields follow, neither compared nor shown: ``_validated_for`` = the ``(Sk, BLOCK_K)`` these lists
-    have been checked against (set by the functions of this module, whose lists fit by construction, and by
-    ``sparse_attention`` after it has checked a caller-built object once), and ``_retiled`` = the lists of the same
+    Two book-keeping fields follow, neither compared nor shown: ``_validated_for`` = :func:`validation_key` of the
+    ``(Sk, BLOCK_K)`` these lists have been checked against (set by the functions of this module, whose lists fit by
+    construction, and by ``sparse_attention`` after it has checked a caller-built object; the key carries the address
+    and the in-place version counter of the four list tensors, so lists edited in place or replaced are checked
+    again), and ``_retiled`` = the lists of the same
     mask at tile sizes the kernels have, kept by ``sparse_attention`` when it was asked for sizes they do not have.
     """
 
@@ -48,8 +50,16 @@ class MaskMetadata:
     packed_masks: Optional[torch.Tensor] = None
     schedule: Optional[torch.Tensor] = None
     schedule_mode: int = 0
-    _validated_for: Optional[Tuple[int, int]] = field(default=None, repr=False, compare=False)
+    _validated_for: Optional[tuple] = field(default=None, repr=False, compare=False)
     _retiled: Optional[tuple] = field(default=None, repr=False, compare=False)
+
+
+def validation_key(md, Sk: int, BLOCK_K: int) -> tuple:
+    """What "these lists were checked against Sk and BLOCK_K" is remembered under: the sizes plus, per list tensor,
+    its address and torch's in-place version counter (shared by all views of a storage), so that an in-place edit
+    of the lists or other tensors under the same object make the remembered check void."""
+    return (int(Sk), int(BLOCK_K)) + tuple(
+        (t.data_ptr(), t._version) for t in (md.unmasked_kv_ids, md.unmasked_lens, md.masked_kv_ids, md.masked_lens))
 
 
 def _check_mask(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int):
@@ -185,7 +195,7 @@ def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int, pack_par
             packed = packed.expand(B, H, nQ, nK, BLOCK_Q * BLOCK_K // 8)
         sched, mode = _make_schedule(lib, fl, pl, B, H, Sq, Sk, BLOCK_Q, BLOCK_K, schedule, dev)
     md = MaskMetadata(fid, fl, pid, pl, packed, sched, mode)
-    md._validated_for = (int(Sk), int(BLOCK_K))  # lists made by the kernels above fit these sizes by construction
+    md._validated_for = validation_key(md, Sk, BLOCK_K)  # lists made by the kernels above fit by construction
     return md
 
 
@@ -432,5 +442,5 @@ def compute_mask_terms(terms: Sequence[MaskTerm], B: int, H: int, Sq: int, Sk: i
         del workspace
         sched, mode = _make_schedule(lib, fl, pl, B, H, Sq, Sk, BLOCK_Q, BLOCK_K, schedule, dev)
     md = MaskMetadata(fid, fl, pid, pl, packed, sched, mode)
-    md._validated_for = (int(Sk), int(BLOCK_K))  # lists made by the kernels above fit these sizes by construction
+    md._validated_for = validation_key(md, Sk, BLOCK_K)  # lists made by the kernels above fit by construction
     return md

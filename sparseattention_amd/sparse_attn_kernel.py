@@ -6,7 +6,7 @@ import math
 import torch
 
 from . import _native
-from .mask_utils import MaskMetadata, Tiling, compute_mask_kernel, compute_mask_terms
+from .mask_utils import MaskMetadata, Tiling, compute_mask_kernel, compute_mask_terms, validation_key
 
 _DTYPES = {torch.bfloat16: _native.SA_DTYPE_BF16, torch.float16: _native.SA_DTYPE_FP16}
 # the forward also takes float32 (a plain kernel on the vector units, for checks against fp32 references)
@@ -73,9 +73,10 @@ def validate_metadata(md: MaskMetadata, Sk: int, BLOCK_K: int) -> None:
 
 
 def _checked_metadata(md: MaskMetadata, Sk: int, BLOCK_K: int) -> None:
-    """validate_metadata once per (object, tiling); metadata made by compute_mask_kernel / compute_mask_terms is
-    trusted (marked there), so the usual call path never synchronises."""
-    key = (int(Sk), int(BLOCK_K))
+    """validate_metadata once per (object, tiling, state of its list tensors); metadata made by compute_mask_kernel /
+    compute_mask_terms is trusted (marked there), so the usual call path never synchronises.  Lists edited in place
+    afterwards, or an object whose tensors were exchanged (dataclasses.replace, copy), are checked again."""
+    key = validation_key(md, Sk, BLOCK_K)
     if getattr(md, "_validated_for", None) == key:
         return
     validate_metadata(md, Sk, BLOCK_K)

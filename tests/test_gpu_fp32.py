@@ -95,3 +95,33 @@ def test_c_abi_limits_of_float32(gpu):
     # the wrapper runs the same request on tiles the kernel has
     o = sparse_attention(q, q, q, mask, 256, 32)
     assert torch.equal(o, torch.zeros_like(q))
+
+
+@pytest.mark.parametrize("D,BQ,BK", [(64, 48, 24), (64, 64, 40), (128, 32, 96), (128, 256, 32), (64, 8, 24)])
+def test_tile_widths_that_are_no_power_of_two_and_the_widest_tile(gpu, D, BQ, BK):
+    # BLOCK_K not a multiple of 32 ends every tile in a partial 32-key step; both mask sources; D = 128 at 256-row tiles
+    B, H, S = 1, 2, 960 if BK in (24, 40, 96) else 512
+    q, k, v = W.qkv(B, H, S, D, torch.float32, seed=BQ + BK)
+    mask = W.random_block_mask(S, 16, 0.5, seed=BK, partial_fraction=0.3)
+    want = sdpa_cpu(q, k, v, mask)
+    me = mask.to(gpu)[None, None].expand(B, H, S, S)
+    lib = _native.load()
+    st = _native.strides
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    md_all = compute_mask_kernel(me, BQ, BK, pack_partial=BK % 8 == 0)
+    for packed in ([None, md_all.packed_masks] if BK % 8 == 0 else [None]):
+        o = torch.full_like(qg, float("nan"))
+        rc = lib.sa_sparse_attention_fwd_ex(
+            qg.data_ptr(), st(qg.stride()), kg.data_ptr(), st(kg.stride()), vg.data_ptr(), st(vg.stride()), o.data_ptr(),
+            st(o.stride()), me.data_ptr(), st(me.stride()),
+            md_all.unmasked_kv_ids.data_ptr(), st(md_all.unmasked_kv_ids.stride()), md_all.unmasked_lens.data_ptr(),
+            st(md_all.unmasked_lens.stride()), md_all.masked_kv_ids.data_ptr(), st(md_all.masked_kv_ids.stride()),
+            md_all.masked_lens.data_ptr(), st(md_all.masked_lens.stride()),
+            packed.data_ptr() if packed is not None else None, st(packed.stride()[:2]) if packed is not None else None,
+            None, 0, 0, B, H, S, S, D, BQ, BK, _native.SA_DTYPE_FP32, D ** -0.5 / math.log(2),
+            torch.cuda.current_stream().cuda_stream)
+        _native.check(rc)
+        torch.cuda.synchronize()
+        assert (o.cpu() - want).abs().max() <= TOL32, f"packed={packed is not None}"
+        ref = oracle.forward(q.numpy(), k.numpy(), v.numpy(), mask.numpy()[None, None], BQ, BK, p_round=0)
+        assert np.abs(o.cpu().numpy() - ref).max() <= TOL32

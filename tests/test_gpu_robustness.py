@@ -12,6 +12,7 @@ from helpers import assert_metadata_equal
 from sparseattention_amd import (MaskMetadata, _native, compute_backward_metadata, compute_mask_kernel,
                                  compute_mask_slow, sparse_attention, sparse_attention_backward,
                                  sparse_attention_decode, workloads as W)
+from sparseattention_amd.mask_utils import validation_key
 from sparseattention_amd.sparse_attn_kernel import merge_attention_parts, validate_metadata
 
 pytestmark = pytest.mark.gpu
@@ -67,6 +68,12 @@ def test_metadata_that_does_not_fit_is_refused_by_the_wrappers(gpu):
     long.masked_lens[0, 0, 0] = S // BK + 1
     with pytest.raises(ValueError, match="counts"):
         sparse_attention(q, k, v, mask, BQ, BK, mask_metadata=long)
+    # an object that passed once is checked again after an in-place edit of its lists
+    edited = clone(good)
+    sparse_attention(q, k, v, mask, BQ, BK, mask_metadata=edited)
+    edited.masked_lens[0, 0, 0] = S // BK + 1
+    with pytest.raises(ValueError, match="counts"):
+        sparse_attention(q, k, v, mask, BQ, BK, mask_metadata=edited)
     # lists made for a longer Sk: indices past this Sk
     other = compute_mask_kernel(torch.ones(1, 1, S, 2 * S, dtype=torch.bool, device=gpu), BQ, BK, pack_partial=False)
     with pytest.raises(ValueError):
@@ -142,22 +149,22 @@ def _tiles_mask(ids, lens, qt, BQ, BK, S, dev):
     return out.expand(B, H, BQ, S)
 
 
-def test_decode_and_backward_stay_inside_their_tensors_with_lists_that_do_not_fit(gpu):
-    # C ABI, counts beyond the row of tiles and indices out of range: the kernels clamp both (results are then those
-    # of other tiles, as with the reference's masked loads), every access stays inside K, V and the mask.
+def test_decode_clamps_lists_that_do_not_fit(gpu):
+    # C ABI, counts beyond the row of tiles and indices out of range: the decode kernels clamp both (counts to the nKt
+    # tiles of the row, indices into [0, nKt)), so the result is attention over the CLAMPED lists, tiles repeated as
+    # often as they are listed.  That value is formed here from the lists on the host and compared.
     lib = _native.load()
     S = _native.strides
     B, H, Sq, Sk, D, BK = 1, 2, 8, 1024, 64, 32
+    nKt = Sk // BK
     q, k, v = W.qkv(B, H, Sq, D, torch.bfloat16, seed=4, device=gpu, Sk=Sk)
     mask = (torch.rand(Sq, Sk, generator=torch.Generator().manual_seed(4)) < 0.5).to(gpu)
     me = mask[None, None].expand(B, H, Sq, Sk)
-    md = compute_mask_kernel(me, Sq, BK, pack_partial=False)
-    fid, pid = md.unmasked_kv_ids.contiguous().clone(), md.masked_kv_ids.contiguous().clone()
-    fl, pl = md.unmasked_lens.contiguous().clone(), md.masked_lens.contiguous().clone()
-    fid[:] = 1 << 27
+    fid = torch.full((B, H, 1, nKt), 1 << 27, dtype=torch.int32, device=gpu)
+    pid = ((3 * torch.arange(nKt, dtype=torch.int32, device=gpu)) % nKt).expand(B, H, 1, nKt).contiguous()
     pid[..., 1::2] = -3
-    fl[:] = 7
-    pl[:] = Sk // BK + 9
+    fl = torch.full((B, H, 1), 7, dtype=torch.int32, device=gpu)
+    pl = torch.full((B, H, 1), nKt + 9, dtype=torch.int32, device=gpu)
     o = torch.empty_like(q)
     rc = lib.sa_sparse_attention_decode(
         q.data_ptr(), S(q.stride()), k.data_ptr(), S(k.stride()), v.data_ptr(), S(v.stride()), o.data_ptr(), S(o.stride()),
@@ -166,27 +173,111 @@ def test_decode_and_backward_stay_inside_their_tensors_with_lists_that_do_not_fi
         1, None, 0, None, None, torch.cuda.current_stream().cuda_stream)
     _native.check(rc)
     torch.cuda.synchronize()
-    assert not torch.isnan(o).any()
+    # host arithmetic of the clamp: F = 7 FULL entries, all tile nKt - 1; then nKt - 7 PARTIAL entries
+    F_, P_ = 7, min(nKt + 9, nKt - 7)
+    tiles = [(nKt - 1, False)] * F_ + [(min(max(int(t), 0), nKt - 1), True) for t in pid[0, 0, 0, :P_].tolist()]
+    cols = torch.cat([torch.arange(t * BK, (t + 1) * BK, device=gpu) for t, _ in tiles])
+    keep = torch.cat([mask[:, t * BK:(t + 1) * BK] if part else torch.ones(Sq, BK, dtype=torch.bool, device=gpu)
+                      for t, part in tiles], dim=1)
+    want = sdpa32(q, k[:, :, cols], v[:, :, cols], keep)
+    assert (o.float() - want).abs().max() <= TOL
 
-    # backward: valid lists first (the expected gradients), then the same call with corrupted copies
-    B, H, S, D = 1, 2, 256, 64
+
+def _tile_weights(md, packed_source, mask_rc, R, C, nR, nS, dev):
+    """[R, C] float: how often the lists of plane (0, 0) of `md` (resident tiles of 128 rows, streamed tiles of 64
+    columns, counts and indices clamped as the backward kernels clamp them) attend to each entry of `mask_rc`.
+    packed_source: None = PARTIAL entries read the mask at the (clamped) tile they name; else the int ids tensor the
+    packed tiles were made from: slot s carries the entries of the tile that slot named THEN."""
+    Wt = torch.zeros(R, C, device=dev)
+    for rt in range(nR):
+        F_ = min(max(int(md.unmasked_lens[0, 0, rt]), 0), nS)
+        P_ = min(max(int(md.masked_lens[0, 0, rt]), 0), nS - F_)
+        rows = slice(128 * rt, 128 * rt + 128)
+        for e in range(F_):
+            t = min(max(int(md.unmasked_kv_ids[0, 0, rt, e]), 0), nS - 1)
+            Wt[rows, 64 * t:64 * t + 64] += 1.0
+        for e in range(P_):
+            t = min(max(int(md.masked_kv_ids[0, 0, rt, e]), 0), nS - 1)
+            src = t if packed_source is None else int(packed_source[0, 0, rt, e])
+            Wt[rows, 64 * t:64 * t + 64] += mask_rc[rows, 64 * src:64 * src + 64].float()
+    return Wt
+
+
+@pytest.mark.parametrize("pack", [False, True])
+def test_backward_clamps_lists_that_do_not_fit(gpu, pack):
+    # Counts beyond the row of tiles, negative counts and indices out of range, straight to the kernels: they clamp
+    # both, so each pass computes the gradient terms of the CLAMPED lists (tiles repeated as listed; with packed tiles a
+    # slot keeps the entries it was packed with).  Expected values from those lists by host arithmetic + dense fp32.
+    B, H, S, D = 1, 1, 256, 64
     q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=5, device=gpu)
-    mask = W.causal_mask(S, gpu)[None, None].expand(B, H, S, S)
+    m2 = W.causal_mask(S, gpu)
+    mask = m2[None, None].expand(B, H, S, S)
     o, lse = sparse_attention(q, k, v, mask, 128, 32, return_lse=True)
     do = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(6)).to(gpu, torch.bfloat16)
-    bmd = compute_backward_metadata(mask, pack_partial=False)
-    good = sparse_attention_backward(do, q, k, v, o, lse, mask, bmd)
+    bmd = compute_backward_metadata(mask, pack_partial=pack)
+    nR, nS = S // 128, S // 64
+    packed_from = []
     for md in (bmd.by_query, bmd.by_key):
         for name in ("unmasked_kv_ids", "unmasked_lens", "masked_kv_ids", "masked_lens"):
             setattr(md, name, getattr(md, name).contiguous().clone())
-        md.unmasked_kv_ids[..., 0] = 1 << 25
+        packed_from.append(md.masked_kv_ids.clone())
+        md.unmasked_kv_ids[:] = torch.tensor([1 << 25, 1, -7, 2], dtype=torch.int32, device=gpu)
+        md.unmasked_lens[:] = torch.tensor([3, 1 << 16], dtype=torch.int32, device=gpu)
+        # (every causal tile row at 128 x 64 has two PARTIAL tiles, so slots 0 and 1 of `packed` are filled)
         md.masked_kv_ids[..., 0] = -1
-        md.unmasked_lens[:] = 1 << 16
-        md.masked_lens[:] = -4
-        md._validated_for = (S, 64)  # straight to the kernels
-    got = sparse_attention_backward(do, q, k, v, o, lse, mask, bmd)
+        md.masked_kv_ids[..., 1] = 9
+        md.masked_lens[:] = torch.tensor([2, -4], dtype=torch.int32, device=gpu)
+        md._validated_for = validation_key(md, S, 64)  # straight to the kernels
+    got = sparse_attention_backward(do, q, k, v, o, lse, None if pack else mask, bmd)
     torch.cuda.synchronize()
-    assert all(g.shape == w.shape for g, w in zip(got, good))
+    Wq = _tile_weights(bmd.by_query, packed_from[0] if pack else None, m2, S, S, nR, nS, gpu)
+    Wk = _tile_weights(bmd.by_key, packed_from[1] if pack else None, m2.t(), S, S, nR, nS, gpu).t()
+    scale = D ** -0.5
+    q32, k32, v32, o32, do32 = (t[0, 0].float() for t in (q, k, v, o, do))
+    P = torch.exp(q32 @ k32.t() * scale - lse[0, 0][:, None])
+    dS = P * (do32 @ v32.t() - (do32 * o32).sum(-1, keepdim=True))
+    want = (scale * (Wq * dS) @ k32, scale * (Wk * dS).t() @ q32, (Wk * P).t() @ do32)
+    for g, w, name in zip(got, want, ("dq", "dk", "dv")):
+        ref = max(1.0, float(w.abs().max()))
+        err = float((g[0, 0].float() - w).abs().max()) / ref
+        assert err <= TOL, f"{name} off by {err:.3e} of its scale {ref:.2f}"
+
+
+def test_pack_skips_list_entries_that_do_not_fit(gpu):
+    # sa_mask_pack_partial with a caller's own lists: a count beyond the row of tiles is clamped to it and a slot whose
+    # index is outside [0, nK) is left untouched, so nothing outside the mask is read and nothing outside `packed` is
+    # written (guard planes on both sides of the buffer stay as they were).
+    lib = _native.load()
+    S_ = _native.strides
+    S, BQ, BK = 512, 128, 32
+    nQ, nK, tb = S // BQ, S // BK, BQ * BK // 8
+    mask = W.random_block_mask(S, 32, 0.5, seed=21, device=gpu, partial_fraction=0.4)[None, None]
+    md = compute_mask_kernel(mask, BQ, BK, pack_partial=True)
+    want = md.packed_masks.contiguous().clone()
+    ids = md.masked_kv_ids.contiguous().clone()
+    lens = md.masked_lens.contiguous().clone()
+    n0 = int(lens[0, 0, 0])
+    assert n0 >= 2
+    pos = torch.arange(nK, device=gpu)
+    ids[pos.expand_as(ids) >= lens[..., None]] = 1 << 28      # what torch.empty may have left past the counts
+    ids[0, 0, 0, 1] = nK + 5                                   # inside the count, outside the mask
+    ids[0, 0, 1, 0] = -2
+    lens[0, 0, 0] = nK + 1000                                  # count beyond the row of tiles
+    lens[0, 0, 2] = -3                                         # negative count: nothing to pack
+    guard = torch.full((3, nQ, nK, tb), 0xA5, dtype=torch.uint8, device=gpu)
+    packed = guard[1:2].unsqueeze(0)
+    rc = lib.sa_mask_pack_partial(mask.data_ptr(), S_(mask.stride()), 1, 1, S, S, BQ, BK, ids.data_ptr(), S_(ids.stride()),
+                                  lens.data_ptr(), S_(lens.stride()), packed.data_ptr(), S_((0, 0)),
+                                  torch.cuda.current_stream().cuda_stream)
+    _native.check(rc)
+    torch.cuda.synchronize()
+    assert (guard[0] == 0xA5).all() and (guard[2] == 0xA5).all()
+    got = guard[1]
+    assert torch.equal(got[0, 0], want[0, 0, 0, 0]) and (got[0, 1] == 0xA5).all()      # slot 1 skipped
+    assert torch.equal(got[0, 2:n0], want[0, 0, 0, 2:n0]) and (got[0, n0:] == 0xA5).all()
+    assert (got[1, 0] == 0xA5).all() and (got[2] == 0xA5).all()
+    n3 = int(lens[0, 0, 3])
+    assert torch.equal(got[3, :n3], want[0, 0, 3, :n3])
 
 
 def test_decode_route_with_default_metadata(gpu):
