@@ -98,6 +98,12 @@ def parse():
     ap.add_argument("--no-backward", action="store_true", help="skip the backward-pass timing")
     ap.add_argument("--no-long", action="store_true", help="skip the forward on the documents and composed configurations")
     ap.add_argument("--no-tiles", action="store_true", help="skip the timing of the tile-size candidates")
+    ap.add_argument("--power-trace", type=float, default=0.0, metavar="SECONDS",
+                    help="instead of the benchmark: run each forward workload (and a device copy, a library GEMM) for "
+                         "SECONDS without a gap while a child process, started before this one touches the GPU, samples "
+                         "socket power, power cap, engine clock and temperatures from the amdgpu hwmon / sysfs files; "
+                         "prints one JSON line with the figures per workload")
+    ap.add_argument("--power-sampler", default=None, metavar="FILE", help=argparse.SUPPRESS)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy a few times, so that a counter run over this command "
                          "holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -453,8 +459,120 @@ def cpu_baselines():
     return out
 
 
+def power_sampler(path):
+    """The child of --power-trace: never touches the GPU runtime, reads the amdgpu driver's files every 10 ms and
+    appends `time power_W cap_W sclk_MHz junction_C mem_C` lines to `path` until `path + ".stop"` exists."""
+    import glob
+
+    dev = sorted(glob.glob("/sys/class/drm/card*/device"))
+    dev = [d for d in dev if glob.glob(d + "/hwmon/hwmon*/power1_input")]
+    if not dev:
+        open(path, "w").write("no amdgpu hwmon files\n")
+        return
+    dev = dev[0]
+    hw = glob.glob(dev + "/hwmon/hwmon*")[0]
+
+    def rd(f, default="0"):
+        try:
+            with open(f) as fh:
+                return fh.read()
+        except OSError:
+            return default
+
+    def sclk():
+        for line in rd(dev + "/pp_dpm_sclk", "").splitlines():
+            if line.rstrip().endswith("*"):
+                return float(line.split(":")[1].lower().replace("mhz", "").replace("*", ""))
+        return 0.0
+
+    with open(path, "w") as out:
+        while not os.path.exists(path + ".stop"):
+            out.write("%.4f %.1f %.1f %.0f %.1f %.1f\n" % (
+                time.time(), float(rd(hw + "/power1_input")) / 1e6, float(rd(hw + "/power1_cap")) / 1e6, sclk(),
+                float(rd(hw + "/temp2_input")) / 1e3, float(rd(hw + "/temp3_input")) / 1e3))
+            out.flush()
+            time.sleep(0.01)
+
+
+def power_trace(seconds):
+    """Every workload SECONDS long without a gap between launches, under the sampler; per workload the mean launch
+    time over the second half (the settled state) and the sampler's readings over the same span."""
+    import subprocess
+    import tempfile
+
+    tmp = tempfile.mkdtemp(prefix="sa_power_")
+    path = os.path.join(tmp, "samples.txt")
+    child = subprocess.Popen([sys.executable, os.path.abspath(__file__), "--power-sampler", path])
+    time.sleep(0.5)  # idle readings first
+    import torch
+    from sparseattention_amd import compute_mask_kernel, sparse_attention, workloads as W
+
+    torch.cuda.set_device(0)
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=0, device="cuda")
+    spans = []
+
+    def sustained(name, fn, flop):
+        torch.cuda.synchronize()
+        t0 = time.time()
+        n = 0
+        half = None
+        while time.time() - t0 < seconds:
+            for _ in range(25):
+                fn()
+            torch.cuda.synchronize()
+            n += 25
+            if half is None and time.time() - t0 >= seconds / 2:
+                half = (time.time(), n)
+        t1 = time.time()
+        spans.append({"workload": name, "t0": half[0], "t1": t1, "ms_per_launch": round((t1 - half[0]) / (n - half[1]) * 1e3, 4),
+                      "executed_flop": flop})
+        time.sleep(0.3)  # (a gap in the samples between workloads)
+
+    masks = [("causal", W.causal_mask(S, "cuda")), ("dense", torch.ones(S, S, dtype=torch.bool, device="cuda")),
+             ("random blocks p=0.9", W.random_block_mask(S, 128, 0.9, seed=90, device="cuda")),
+             ("no tile attended (q read, zeros written)", torch.zeros(S, S, dtype=torch.bool, device="cuda"))]
+    for name, m in masks:
+        me = m[None, None].expand(B, H, S, S)
+        md = compute_mask_kernel(me, BQ, BK)
+        tiles = int(md.unmasked_lens[0, 0].sum()) + int(md.masked_lens[0, 0].sum())
+        sustained("forward, " + name, lambda: sparse_attention(q, k, v, me, BQ, BK, mask_metadata=md), tiles * B * H * FLOP_PER_TILE)
+    src = torch.ones(1 << 28, dtype=torch.int32, device="cuda")
+    dst = torch.empty_like(src)
+    sustained("device copy 1 GiB (torch)", lambda: dst.copy_(src), 0)
+    del src, dst
+    a = torch.randn(8192, 8192, device="cuda", dtype=torch.bfloat16)
+    bm = torch.randn(8192, 8192, device="cuda", dtype=torch.bfloat16)
+    sustained("bf16 GEMM 8192^3 (torch / hipBLASLt)", lambda: a @ bm, 2 * 8192 ** 3)
+    open(path + ".stop", "w").close()
+    child.wait(timeout=10)
+    rows = [tuple(float(x) for x in ln.split()) for ln in open(path).read().splitlines() if ln[:1].isdigit()]
+    idle = [r for r in rows if r[0] < rows[0][0] + 0.4] if rows else []
+    out = {"power_trace_seconds_per_workload": seconds, "samples": len(rows),
+           "idle": {"power_W": round(sum(r[1] for r in idle) / max(1, len(idle)), 1)} if idle else None, "workloads": []}
+    for sp in spans:
+        rs = [r for r in rows if sp["t0"] <= r[0] <= sp["t1"]]
+        n = max(1, len(rs))
+        tf = sp["executed_flop"] / (sp["ms_per_launch"] * 1e-3) / 1e12 if sp["executed_flop"] else None
+        pw = sum(r[1] for r in rs) / n
+        out["workloads"].append({
+            "workload": sp["workload"], "ms_per_launch": sp["ms_per_launch"],
+            "executed_tflops": round(tf, 1) if tf else None, "samples": len(rs),
+            "power_W_mean": round(pw, 1), "power_W_max": round(max((r[1] for r in rs), default=0.0), 1),
+            "power_cap_W": round(rs[0][2], 1) if rs else None,
+            "sclk_MHz_mean": round(sum(r[3] for r in rs) / n, 0), "sclk_MHz_min": min((r[3] for r in rs), default=0.0),
+            "junction_C_max": max((r[4] for r in rs), default=0.0), "mem_C_max": max((r[5] for r in rs), default=0.0),
+            "W_per_executed_tflops": round(pw / tf, 3) if tf else None})
+    print(json.dumps(out))
+
+
 def main():
     args = parse()
+    if args.power_sampler:
+        power_sampler(args.power_sampler)
+        return
+    if args.power_trace > 0:
+        power_trace(args.power_trace)
+        return
     if args.gpus != 1:
         print(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); the path has no multi-GPU leg.",
               file=sys.stderr)

@@ -303,6 +303,36 @@ int sa_sparse_attention_fwd_lse(const void *q, const int64_t q_strides[4], const
                                 int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2, void *stream);
 
 /*
+ * sa_sparse_attention_fwd_lse (without a schedule) with the choice of the kernel that runs it.  No counterpart in the
+ * reference, whose one kernel is tuned by Triton's autotuner over eight configurations at its first call
+ * (sparse_attn_kernel.py:66-72); here the caller, who knows the mask, chooses.
+ *
+ *   SA_FWD_KERNEL_DEFAULT      what sa_sparse_attention_fwd runs: two workgroups per compute unit, 64 keys per step;
+ *                              the fastest form for lists of some tens of KV tiles and more.
+ *   SA_FWD_KERNEL_SHORT_LISTS  three workgroups per compute unit, 32 keys per step, K/V requested two steps ahead:
+ *                              for masks that leave a Q tile few KV tiles (a Q tile then spends much of its life
+ *                              waiting for its first loads, which a third resident workgroup covers).  Needs bf16 or
+ *                              fp16, D = 128, BQ = 128 and the packed PARTIAL tiles (else SA_ERR_UNSUPPORTED), and it
+ *                              reads at most SA_FWD_SHORT_LISTS_MAX_ENTRIES entries of a Q tile's two lists taken
+ *                              together (FULL entries first): the caller must know that no list is longer, e.g. from
+ *                              the counts of sa_mask_classify.
+ * Both compute the same function; their results differ by rounding only (the keys meet the online softmax in other
+ * groupings).
+ */
+enum sa_fwd_kernel { SA_FWD_KERNEL_DEFAULT = 0, SA_FWD_KERNEL_SHORT_LISTS = 1 };
+#define SA_FWD_SHORT_LISTS_MAX_ENTRIES 256
+int sa_sparse_attention_fwd_kernel(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                                   const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
+                                   const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
+                                   const int64_t full_ids_strides[4], const int32_t *full_lens,
+                                   const int64_t full_lens_strides[3], const int32_t *part_ids,
+                                   const int64_t part_ids_strides[4], const int32_t *part_lens,
+                                   const int64_t part_lens_strides[3], const uint8_t *packed,
+                                   const int64_t packed_strides[2], float *lse, const int64_t lse_strides[3], int B,
+                                   int H, int Sq, int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2,
+                                   int kernel, void *stream);
+
+/*
  * The forward for few query rows against a long K/V (decode): Sq <= 32 rows form the single Q tile of every (b, h),
  * BLOCK_Q = Sq.  The result is that of sparse_attention (sparseattention/sparse_attn_kernel.py:149-185) called with
  * BLOCK_Q = Sq; the reference has no kernel of its own for this shape ("Backwards pass + decode kernels" is item 3

@@ -14,7 +14,8 @@ The device work is done by hand-written gfx950 HIP kernels in ``libsparseattn_hi
 behind the C ABI of ``include/sparseattn.h``.
 """
 from .mask_utils import (MaskMetadata, MaskTerm, block_term, causal_term, compute_mask_kernel, compute_mask_slow,
-                         compute_mask_terms, materialize_mask_terms, select_block_sizes, select_tiling, Tiling)
+                         compute_mask_terms, materialize_mask_terms, select_block_sizes, select_tiling, Tiling,
+                         with_list_stats)
 from .sparse_attn_kernel import (BackwardMetadata, compute_backward_metadata, compute_backward_metadata_terms,
                                  merge_attention_parts, sparse_attention,
                                  sparse_attention_backward, sparse_attention_decode, sparse_attention_kv_split,
@@ -24,4 +25,4 @@ __all__ = ["MaskMetadata", "compute_mask_kernel", "compute_mask_slow", "select_b
            "sparse_attention_decode", "sparse_attention_backward", "sparse_attention_trainable", "BackwardMetadata",
            "compute_backward_metadata", "merge_attention_parts", "sparse_attention_kv_split", "MaskTerm", "causal_term",
            "block_term", "compute_mask_terms", "materialize_mask_terms", "compute_backward_metadata_terms", "select_tiling",
-           "Tiling", "sparse_attention_tiled"]
+           "Tiling", "sparse_attention_tiled", "with_list_stats"]

@@ -23,6 +23,9 @@ SA_DTYPE_FP32 = 2  # forward only
 
 SA_SCHEDULE_PERSISTENT = 0
 SA_SCHEDULE_PAIRS = 1
+SA_FWD_KERNEL_DEFAULT = 0
+SA_FWD_KERNEL_SHORT_LISTS = 1
+SA_FWD_SHORT_LISTS_MAX_ENTRIES = 256
 
 #: every symbol include/sparseattn.h declares
 EXPORTS = (
@@ -39,6 +42,7 @@ EXPORTS = (
     "sa_fwd_schedule",
     "sa_sparse_attention_fwd_ex",
     "sa_sparse_attention_fwd_lse",
+    "sa_sparse_attention_fwd_kernel",
     "sa_decode_num_splits",
     "sa_decode_workspace_bytes",
     "sa_sparse_attention_decode",
@@ -115,6 +119,11 @@ def load() -> ctypes.CDLL:
     lib.sa_decode_workspace_bytes.restype = ctypes.c_size_t
     lib.sa_decode_workspace_bytes.argtypes = [ctypes.c_int] * 5
     lib.sa_sparse_attention_decode.restype = ctypes.c_int
+    lib.sa_sparse_attention_fwd_kernel.restype = ctypes.c_int
+    lib.sa_sparse_attention_fwd_kernel.argtypes = (
+        [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] + [ctypes.c_int] * 8
+        + [ctypes.c_float, ctypes.c_int, _vp]
+    )
     lib.sa_sparse_attention_decode.argtypes = (
         [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [ctypes.c_int] * 7 + [ctypes.c_float, ctypes.c_int]
         + [_vp, ctypes.c_size_t] + [_vp, _i64p] + [_vp]

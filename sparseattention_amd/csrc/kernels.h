@@ -128,6 +128,11 @@ struct FwdParams {
 
 // dtype: 0 bf16, 1 fp16.  Returns hipErrorInvalidValue when no instantiation matches (D, BQ).
 hipError_t launch_fwd(const FwdParams &p, int dtype, int D, int BQ, hipStream_t stream);
+// The forward for short lists (sparse_fwd_c32.hip): three workgroups per compute unit, 32 keys per step.  It exists
+// for bf16 / fp16, D = 128, BLOCK_Q = 128, bit-packed PARTIAL tiles, no schedule (fwd_c32_has), and cuts lists at
+// 256 entries.  Results agree with launch_fwd within rounding (the keys meet the online softmax in other groupings).
+bool fwd_c32_has(const FwdParams &p, int dtype, int D, int BQ);
+hipError_t launch_fwd_c32(const FwdParams &p, int dtype, int D, int BQ, hipStream_t stream);
 // float32 q, k, v, o (the pointers of FwdParams then address floats; strides stay in elements): any BQ from 1 to 256
 // (to 128 at D = 256), any BK; reads the packed tiles when given, else the mask; no schedules.
 hipError_t launch_fwd_f32(const FwdParams &p, int D, int BQ, hipStream_t stream);

@@ -246,8 +246,11 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
                  const int64_t part_ids_strides[4], const int32_t *part_lens, const int64_t part_lens_strides[3],
                  const uint8_t *packed, const int64_t packed_strides[2], bool use_packed, const int32_t *schedule,
                  size_t schedule_bytes, int schedule_mode, float *lse, const int64_t lse_strides[3], int B, int H,
-                 int Sq, int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2, void *stream) {
+                 int Sq, int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2, void *stream,
+                 int kernel = SA_FWD_KERNEL_DEFAULT) {
     g_error[0] = 0;
+    if (kernel != SA_FWD_KERNEL_DEFAULT && kernel != SA_FWD_KERNEL_SHORT_LISTS)
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd_kernel: kernel %d (0 = default, 1 = short lists)", kernel);
     if (!q || !k || !v || !o || !q_strides || !k_strides || !v_strides || !o_strides || !full_ids ||
         !full_ids_strides || !full_lens || !full_lens_strides || !part_ids || !part_ids_strides || !part_lens ||
         !part_lens_strides)
@@ -357,6 +360,15 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
         fp.lse = lse;
         for (int i = 0; i < 3; i++) fp.lses[i] = lse_strides[i];
     }
+    if (kernel == SA_FWD_KERNEL_SHORT_LISTS) {
+        if (f32 || !sa::fwd_c32_has(fp, dtype, D, BQ))
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd_kernel: the short-list kernel needs bf16 or fp16, head dim 128, BLOCK_Q 128, packed PARTIAL tiles and no schedule");
+        if (Sk / BK > SA_FWD_SHORT_LISTS_MAX_ENTRIES * 64)  // (its packed-slot arithmetic stays inside 32 bits far beyond this)
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd_kernel: Sk/BLOCK_K %d", Sk / BK);
+        const hipError_t e1 = sa::launch_fwd_c32(fp, dtype, D, BQ, static_cast<hipStream_t>(stream));
+        if (e1 != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_fwd_kernel: launch failed: %s", hipGetErrorString(e1));
+        return SA_OK;
+    }
     const hipError_t e = f32 ? sa::launch_fwd_f32(fp, D, BQ, static_cast<hipStream_t>(stream))
                              : sa::launch_fwd(fp, dtype, D, BQ, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_fwd: launch failed: %s", hipGetErrorString(e));
@@ -439,6 +451,29 @@ int sa_sparse_attention_fwd_lse(const void *q, const int64_t q_strides[4], const
                         full_ids_strides, full_lens, full_lens_strides, part_ids, part_ids_strides, part_lens,
                         part_lens_strides, packed, packed_strides, use_packed, schedule, schedule_bytes, schedule_mode,
                         lse, lse_strides, B, H, Sq, Sk, D, BQ, BK, dtype, sm_scale_log2, stream);
+}
+
+int sa_sparse_attention_fwd_kernel(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                                   const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
+                                   const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
+                                   const int64_t full_ids_strides[4], const int32_t *full_lens,
+                                   const int64_t full_lens_strides[3], const int32_t *part_ids,
+                                   const int64_t part_ids_strides[4], const int32_t *part_lens,
+                                   const int64_t part_lens_strides[3], const uint8_t *packed,
+                                   const int64_t packed_strides[2], float *lse, const int64_t lse_strides[3], int B,
+                                   int H, int Sq, int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2,
+                                   int kernel, void *stream) {
+    const bool use_packed = packed != nullptr;
+    if (use_packed) {
+        g_error[0] = 0;
+        if (!packed_strides) return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd_kernel: null pointer argument (packed_strides)");
+        if ((B > 1 && packed_strides[0] % 4) || (H > 1 && packed_strides[1] % 4) || !aligned(packed, 4))
+            return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd_kernel: packed needs a 4-byte aligned base and plane strides");
+    }
+    return forward_impl(q, q_strides, k, k_strides, v, v_strides, o, o_strides, mask, mask_strides, full_ids,
+                        full_ids_strides, full_lens, full_lens_strides, part_ids, part_ids_strides, part_lens,
+                        part_lens_strides, packed, packed_strides, use_packed, nullptr, 0, 0, lse, lse_strides, B, H, Sq,
+                        Sk, D, BQ, BK, dtype, sm_scale_log2, stream, kernel);
 }
 
 int sa_validate_metadata(const int32_t *full_ids, const int64_t full_ids_strides[4], const int32_t *full_lens,

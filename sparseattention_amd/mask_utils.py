@@ -35,6 +35,11 @@ class MaskMetadata:
     ``compute_mask_kernel(..., schedule="pairs" | "persistent")``.  It depends on the counts, on B and H and, for
     "persistent", on the device; without it the forward launches one workgroup per Q tile.
 
+    ``list_stats`` is the third addition (optional, default None): ``(mean, longest)`` number of listed KV tiles per
+    Q tile, FULL and PARTIAL together, as Python numbers.  Reading them back synchronises the host with the device
+    once, so they are filled only on request (``compute_mask_kernel(..., list_stats=True)`` or
+    :func:`with_list_stats`); with them :func:`sparse_attention` picks the kernel form that suits the lists.
+
     Two book-keeping fields follow, neither compared nor shown: ``_validated_for`` = :func:`validation_key` of the
     ``(Sk, BLOCK_K)`` these lists have been checked against (set by the functions of this module, whose lists fit by
     construction, and by ``sparse_attention`` after it has checked a caller-built object; the key carries the address
@@ -50,8 +55,23 @@ class MaskMetadata:
     packed_masks: Optional[torch.Tensor] = None
     schedule: Optional[torch.Tensor] = None
     schedule_mode: int = 0
+    list_stats: Optional[Tuple[float, int]] = None
     _validated_for: Optional[tuple] = field(default=None, repr=False, compare=False)
     _retiled: Optional[tuple] = field(default=None, repr=False, compare=False)
+
+
+def with_list_stats(md: "MaskMetadata") -> "MaskMetadata":
+    """Fills ``md.list_stats`` = (mean, longest) listed KV tiles per Q tile from the two count tensors (one host
+    synchronisation; the distinct planes of broadcast counts are read once) and returns ``md``."""
+    fl, pl = md.unmasked_lens, md.masked_lens
+    idx = tuple(slice(0, 1) if fl.stride(d) == 0 and pl.stride(d) == 0 else slice(None) for d in range(2))
+    total = (fl[idx].to(torch.int64) + pl[idx].to(torch.int64)).flatten()
+    if total.numel() == 0:
+        md.list_stats = (0.0, 0)
+    else:
+        both = torch.stack((total.sum(), total.max())).tolist()
+        md.list_stats = (both[0] / total.numel(), int(both[1]))
+    return md
 
 
 def validation_key(md, Sk: int, BLOCK_K: int) -> tuple:
@@ -128,7 +148,7 @@ def _make_schedule(lib, fl, pl, B, H, Sq, Sk, BLOCK_Q, BLOCK_K, schedule, dev):
 
 
 def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int, pack_partial: Optional[bool] = None,
-                        schedule=None) -> MaskMetadata:
+                        schedule=None, list_stats: bool = False) -> MaskMetadata:
     """Classify the mask's tiles on the GPU (replaces mask_utils.py:85-107).
 
     Memory beyond the reference's four tensors: with ``pack_partial`` (the default when BLOCK_K is a multiple of 8)
@@ -149,6 +169,9 @@ def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int, pack_par
     on MI355X it wins when the lists are short (a few hundred keys per Q tile) and loses a few percent to the
     hardware dispatcher when they are long, because a static hand-out cannot follow the uneven pace of the
     workgroups that share a compute unit.
+    ``list_stats``: also read back how many KV tiles the lists hold per Q tile (mean and longest:
+    ``MaskMetadata.list_stats``), which lets :func:`sparse_attention` choose the kernel form for short lists.  This is
+    the one option that synchronises the host with the device; preprocessing is paid once per mask (README.md:46).
     """
     B, H, Sq, Sk = _check_mask(mask, BLOCK_Q, BLOCK_K)
     if not mask.is_cuda:
@@ -196,7 +219,7 @@ def compute_mask_kernel(mask: torch.Tensor, BLOCK_Q: int, BLOCK_K: int, pack_par
         sched, mode = _make_schedule(lib, fl, pl, B, H, Sq, Sk, BLOCK_Q, BLOCK_K, schedule, dev)
     md = MaskMetadata(fid, fl, pid, pl, packed, sched, mode)
     md._validated_for = validation_key(md, Sk, BLOCK_K)  # lists made by the kernels above fit by construction
-    return md
+    return with_list_stats(md) if list_stats else md
 
 
 # Tile sizes tried by select_block_sizes, and what one executed mask entry costs at each of them relative to tiles of

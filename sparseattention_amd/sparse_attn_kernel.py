@@ -111,8 +111,35 @@ def kernel_tiles(Sq: int, Sk: int, D: int, BLOCK_Q: int, BLOCK_K: int):
     return next(((bq, bk) for bk in (32, 64, 16) if Sk % bk == 0), None)
 
 
+# Below this many listed keys per Q tile (mean over the Q tiles) the forward runs its short-list kernel when the
+# metadata says so (MaskMetadata.list_stats) and the kernel has the sizes.  Measured on MI355X (B8 H32 S4096 D128,
+# tiles 128x32, default / short-list kernel): 448 keys per Q tile 0.343 / 0.340 ms, 1222 keys 0.709 / 0.719 ms,
+# 2100 keys and more +5 ... +8 %: the third workgroup per compute unit pays for itself on the shortest lists only.
+SHORT_LIST_KEYS = 512
+
+
+def _short_list_kernel(mask_metadata, dtype, D, BLOCK_Q, BLOCK_K, kernel) -> bool:
+    """Whether this call runs the kernel for short lists (three workgroups per compute unit, 32 keys per step)."""
+    if kernel not in (None, "auto", "default", "short"):
+        raise ValueError(f"kernel must be 'auto', 'default' or 'short' (got {kernel!r})")
+    if kernel == "default":
+        return False
+    has = (dtype in _DTYPES and D == 128 and BLOCK_Q == 128 and BLOCK_K >= 16 and BLOCK_K & (BLOCK_K - 1) == 0
+           and getattr(mask_metadata, "packed_masks", None) is not None
+           and getattr(mask_metadata, "schedule", None) is None)
+    stats = getattr(mask_metadata, "list_stats", None)
+    fits = stats is not None and stats[1] <= _native.SA_FWD_SHORT_LISTS_MAX_ENTRIES
+    if kernel == "short":
+        if not (has and fits):
+            raise ValueError("kernel='short' needs bf16/fp16, head dim 128, BLOCK_Q 128, mask_metadata with packed_masks, "
+                             "no schedule, and list_stats whose longest list has at most "
+                             f"{_native.SA_FWD_SHORT_LISTS_MAX_ENTRIES} entries")
+        return True
+    return has and fits and stats[0] * BLOCK_K < SHORT_LIST_KEYS
+
+
 def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor | None, BLOCK_Q, BLOCK_K,
-                     mask_metadata: MaskMetadata | None = None, *, return_lse: bool = False):
+                     mask_metadata: MaskMetadata | None = None, *, return_lse: bool = False, kernel: str | None = None):
     """softmax(q kᵀ / sqrt(D) + (mask ? 0 : -inf)) v, skipping KV tiles the mask empties.
 
     Signature and meaning follow sparse_attn_kernel.py:149-185: ``q`` [B,H,Sq,D], ``k``/``v``
@@ -125,6 +152,12 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
     [B,H,Sq] float32 is the log of the row's softmax denominator, -inf for rows that attend to nothing.
     ``mask`` may be None when ``mask_metadata`` carries ``packed_masks`` (the kernels then read no mask tensor), which
     is how masks given by a formula run (:func:`compute_mask_terms`).
+    ``kernel`` (not in the reference, whose one kernel Triton autotunes at the first call, sparse_attn_kernel.py:66-72):
+    "default" = two workgroups per compute unit, 64 keys per step; "short" = the form for masks that leave a Q tile
+    few KV tiles (three workgroups per compute unit, 32 keys per step; bf16/fp16, D = 128, BLOCK_Q = 128, packed
+    PARTIAL tiles, ``mask_metadata.list_stats`` with no list above 256 entries); None / "auto" = "short" when the
+    metadata carries ``list_stats`` (``compute_mask_kernel(..., list_stats=True)``) that say the lists are short,
+    else "default".  The two agree within rounding.
     """
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be [B,H,S,D]")
@@ -224,7 +257,11 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
                 torch.cuda.current_stream(q.device).cuda_stream)
         sched = getattr(mask_metadata, "schedule", None)
         lse = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device) if return_lse else None
-        if packed is not None or sched is not None or return_lse:
+        if _short_list_kernel(mask_metadata, q.dtype, Dk, int(BLOCK_Q), int(BLOCK_K), kernel):
+            rc = lib.sa_sparse_attention_fwd_kernel(
+                *common, packed.data_ptr(), S(packed.stride()[:2]), lse.data_ptr() if return_lse else None,
+                S(lse.stride()) if return_lse else None, *tail[:-1], _native.SA_FWD_KERNEL_SHORT_LISTS, tail[-1])
+        elif packed is not None or sched is not None or return_lse:
             pk = (packed.data_ptr(), S(packed.stride()[:2])) if packed is not None else (None, None)
             sc = ((sched.data_ptr(), sched.numel() * 4, int(getattr(mask_metadata, "schedule_mode", 0)))
                   if sched is not None else (None, 0, 0))
