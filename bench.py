@@ -533,9 +533,37 @@ def power_trace(seconds):
              ("no tile attended (q read, zeros written)", torch.zeros(S, S, dtype=torch.bool, device="cuda"))]
     for name, m in masks:
         me = m[None, None].expand(B, H, S, S)
-        md = compute_mask_kernel(me, BQ, BK)
+        md = compute_mask_kernel(me, BQ, BK, list_stats=True)
         tiles = int(md.unmasked_lens[0, 0].sum()) + int(md.masked_lens[0, 0].sum())
-        sustained("forward, " + name, lambda: sparse_attention(q, k, v, me, BQ, BK, mask_metadata=md), tiles * B * H * FLOP_PER_TILE)
+        flop = tiles * B * H * FLOP_PER_TILE
+        sustained("forward, " + name, lambda: sparse_attention(q, k, v, me, BQ, BK, mask_metadata=md, kernel="default"), flop)
+        if name == "causal":  # the same mask and work through the 256-row kernel (8 waves, one workgroup per CU)
+            md2 = compute_mask_kernel(me, 256, BK)
+            t2 = int(md2.unmasked_lens[0, 0].sum()) + int(md2.masked_lens[0, 0].sum())
+            sustained("forward, causal, tiles 256x32 (8-wave two-phase kernel)",
+                      lambda: sparse_attention(q, k, v, me, 256, BK, mask_metadata=md2), t2 * B * H * 2 * FLOP_PER_TILE)
+        if name.endswith("p=0.9"):
+            sustained("forward, " + name + ", short-list kernel",
+                      lambda: sparse_attention(q, k, v, me, BQ, BK, mask_metadata=md, kernel="short"), flop)
+    # backward of the causal workload (algorithmic flop: five products per executed 128x64 tile)
+    from sparseattention_amd import compute_backward_metadata, sparse_attention_backward, sparse_attention_decode
+
+    me = masks[0][1][None, None].expand(B, H, S, S)
+    bmd = compute_backward_metadata(me)
+    o, lse = sparse_attention(q, k, v, me, BQ, BK, return_lse=True)
+    do = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(3)).to("cuda", torch.bfloat16)
+    tq = int(bmd.by_query.unmasked_lens[0, 0].sum()) + int(bmd.by_query.masked_lens[0, 0].sum())
+    tk = int(bmd.by_key.unmasked_lens[0, 0].sum()) + int(bmd.by_key.masked_lens[0, 0].sum())
+    sustained("backward, causal (algorithmic flop)", lambda: sparse_attention_backward(do, q, k, v, o, lse, me, bmd),
+              (3 * tq + 2 * tk) * 2 * 128 * 64 * D * B * H)
+    del o, lse, do, bmd
+    # decode: one query row against every key of a 32k context (HBM-bound)
+    qd, kd, vd = W.qkv(B, H, 1, D, torch.bfloat16, seed=1, device="cuda", Sk=32768)
+    md_d = compute_mask_kernel(torch.ones(B, H, 1, 32768, dtype=torch.bool, device="cuda"), 1, 128)
+    mk_d = torch.ones(1, 32768, dtype=torch.bool, device="cuda").expand(B, H, 1, 32768)
+    sustained("decode, 1 query row, Sk=32768 (4 GiB of K/V per launch)",
+              lambda: sparse_attention_decode(qd, kd, vd, mk_d, 128, mask_metadata=md_d), 0)
+    del qd, kd, vd
     src = torch.ones(1 << 28, dtype=torch.int32, device="cuda")
     dst = torch.empty_like(src)
     sustained("device copy 1 GiB (torch)", lambda: dst.copy_(src), 0)
