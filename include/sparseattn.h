@@ -316,10 +316,20 @@ int sa_sparse_attention_fwd_lse(const void *q, const int64_t q_strides[4], const
  *                              reads at most SA_FWD_SHORT_LISTS_MAX_ENTRIES entries of a Q tile's two lists taken
  *                              together (FULL entries first): the caller must know that no list is longer, e.g. from
  *                              the counts of sa_mask_classify.
- * Both compute the same function; their results differ by rounding only (the keys meet the online softmax in other
- * groupings).
+ *   SA_FWD_KERNEL_ROTATED_BY(G)  the default kernel, with Q tile qt walking its FULL entries (all but the first chunk
+ *                              of 64 keys) from a start BQ/64 * (G - 1 - qt mod G) chunks further on, wrapping
+ *                              around; 2 <= G <= 64, a power of two (a Q tile whose FULL list is shorter than the
+ *                              largest start halves G until it fits).  For banded masks (sliding windows): the windows of neighbouring Q tiles
+ *                              are BQ keys apart, so walked from the front they read the same K/V rows two chunks
+ *                              apart and find them evicted from L2; walked this way G neighbours read them at the
+ *                              same time.  The reference fixes FULL entries before PARTIAL ones
+ *                              (sparse_attn_kernel.py:113-142), which stays; the order inside the FULL list is its
+ *                              list order there and this rotation of it here.
+ * All compute the same function; their results differ by rounding only (the keys meet the online softmax in other
+ * groupings or another order).
  */
-enum sa_fwd_kernel { SA_FWD_KERNEL_DEFAULT = 0, SA_FWD_KERNEL_SHORT_LISTS = 1 };
+enum sa_fwd_kernel { SA_FWD_KERNEL_DEFAULT = 0, SA_FWD_KERNEL_SHORT_LISTS = 1, SA_FWD_KERNEL_ROTATED = 2 };
+#define SA_FWD_KERNEL_ROTATED_BY(G) (SA_FWD_KERNEL_ROTATED | ((G) << 8))
 #define SA_FWD_SHORT_LISTS_MAX_ENTRIES 256
 int sa_sparse_attention_fwd_kernel(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
                                    const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],

@@ -25,6 +25,7 @@ SA_SCHEDULE_PERSISTENT = 0
 SA_SCHEDULE_PAIRS = 1
 SA_FWD_KERNEL_DEFAULT = 0
 SA_FWD_KERNEL_SHORT_LISTS = 1
+SA_FWD_KERNEL_ROTATED = 2
 SA_FWD_SHORT_LISTS_MAX_ENTRIES = 256
 
 #: every symbol include/sparseattn.h declares

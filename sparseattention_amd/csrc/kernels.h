@@ -120,6 +120,9 @@ struct FwdParams {
     const int32_t *sched;
     int sched_G, sched_R;  // workgroups, and entries per row after the header entry
     float scale;    // softmax scale / ln 2
+    // 0, or the group size G of the rotated walk of the FULL entries (sparse_fwd_kernel, one workgroup per Q tile):
+    // Q tile qt starts 2 * (G - 1 - qt mod G) chunks into its FULL entries.
+    int rot;
     // Optional second output: natural-log sum of exp(scaled score) over the attended keys of every query row
     // (-inf for rows without one), or null.
     float *lse;

@@ -332,9 +332,35 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
         if ((unsigned)idx >= (unsigned)p.nK) return kAbsent;
         return (MODE == 2 ? (idx << p.lbk) : (idx << LBKC)) | (e >= F ? kPartialBit : 0);
     };
+    // Where list entry e goes in the LDS copy.  With p.rot = G > 0 the chunks that hold FULL entries only, but for the
+    // first (requested before the list is copied), are walked from a start that depends on the Q tile: tile qt starts
+    // BQ/64 * (G - 1 - qt mod G) chunks further on, wrapping around.  Neighbouring Q tiles of a banded mask (a sliding
+    // window) have windows BQ keys apart and run at the same time; walked from the front they read the same keys two
+    // chunks apart, with everything the other resident workgroups read in between, and find them gone from L2.
+    // Walked this way G neighbours read the same keys at the same time.  The order inside a list changes the result by
+    // rounding only (sparse_attn_kernel.py:113-142 fixes FULL entries before PARTIAL ones, which stays).
+    const int rot_first = MODE == 2 ? 1 : EPC;                                    // entries of the first chunk
+    const int rot_n = MODE == 2 ? max(F - 1, 0) : max((F / EPC) * EPC - EPC, 0);  // entries that take part
+    int rot_by = 0;
+    if (!PS && p.rot > 0 && rot_n > 0) {
+        // the group shrinks (by halves) until its largest start lies inside the entries that take part: neighbours of a
+        // band have lists of one length, so they agree on it
+        constexpr int CPT = NW >= 2 ? NW / 2 : 1;  // chunks of 64 keys per Q tile height
+        const int n_chunks = MODE == 2 ? (rot_n << (p.lbk - 6)) : rot_n / EPC;
+        int G = p.rot;
+        while (G > 1 && CPT * (G - 1) >= n_chunks) G >>= 1;
+        const int chunks = CPT * (G - 1 - (qt % G));
+        rot_by = (MODE == 2 ? (chunks >> (p.lbk - 6)) : chunks * EPC) % rot_n;
+    }
+    auto list_pos = [&](int e) -> int {
+        if (PS || e < rot_first || e >= rot_first + rot_n) return e;
+        int x = e - rot_first - rot_by;
+        if (x < 0) x += rot_n;
+        return rot_first + x;
+    };
     auto copy_list = [&]() {
         if (list_in_lds) {
-            for (int e = tid; e < list_cnt; e += NW * 64) ent[e] = tagged_entry(e);
+            for (int e = tid; e < list_cnt; e += NW * 64) ent[list_pos(e)] = tagged_entry(e);
         }
     };
     // First key column of every list entry in chunk t (t < T), plus which entries exist / are partial, in two
@@ -1037,9 +1063,9 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
             const bool mine = list_in_lds && tid < list_cnt;
             int first_slots = 0;
             if (mine) first_slots = tagged_entry(tid);
-            if (mine) ent[tid] = first_slots;
+            if (mine) ent[list_pos(tid)] = first_slots;
             if (list_in_lds)
-                for (int e = tid + NW * 64; e < list_cnt; e += NW * 64) ent[e] = tagged_entry(e);
+                for (int e = tid + NW * 64; e < list_cnt; e += NW * 64) ent[list_pos(e)] = tagged_entry(e);
         } else {
             copy_list();
         }

@@ -249,8 +249,11 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
                  int Sq, int Sk, int D, int BQ, int BK, int dtype, float sm_scale_log2, void *stream,
                  int kernel = SA_FWD_KERNEL_DEFAULT) {
     g_error[0] = 0;
-    if (kernel != SA_FWD_KERNEL_DEFAULT && kernel != SA_FWD_KERNEL_SHORT_LISTS)
-        return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd_kernel: kernel %d (0 = default, 1 = short lists)", kernel);
+    const int rot_group = kernel >> 8;
+    kernel &= 0xff;
+    if ((kernel != SA_FWD_KERNEL_DEFAULT && kernel != SA_FWD_KERNEL_SHORT_LISTS && kernel != SA_FWD_KERNEL_ROTATED) ||
+        (kernel == SA_FWD_KERNEL_ROTATED ? (rot_group < 2 || rot_group > 64 || (rot_group & (rot_group - 1))) : rot_group != 0))
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd_kernel: kernel %d, group %d (0 = default, 1 = short lists, SA_FWD_KERNEL_ROTATED_BY(G) with G = 2, 4, ... 64)", kernel, rot_group);
     if (!q || !k || !v || !o || !q_strides || !k_strides || !v_strides || !o_strides || !full_ids ||
         !full_ids_strides || !full_lens || !full_lens_strides || !part_ids || !part_ids_strides || !part_lens ||
         !part_lens_strides)
@@ -352,6 +355,7 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
                        ? 1
                        : 0;
     fp.scale = sm_scale_log2;
+    fp.rot = (kernel == SA_FWD_KERNEL_ROTATED && !f32) ? rot_group : 0;
     fp.lse = nullptr;
     if (lse) {
         if (!lse_strides) return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd_lse: null pointer argument (lse_strides)");

@@ -39,6 +39,10 @@ class MaskMetadata:
     Q tile, FULL and PARTIAL together, as Python numbers.  Reading them back synchronises the host with the device
     once, so they are filled only on request (``compute_mask_kernel(..., list_stats=True)`` or
     :func:`with_list_stats`); with them :func:`sparse_attention` picks the kernel form that suits the lists.
+    ``list_rotation`` comes from the same read-back: a group size G > 0 when the FULL lists of neighbouring Q tiles
+    slide along the keys (a sliding window), for which the forward then walks the FULL entries of Q tile qt from a
+    start that depends on qt, so that neighbours read the same K/V rows at the same time (they are fetched from HBM
+    once instead of once per Q tile); 0 (the default) walks every list from its front.
 
     Two book-keeping fields follow, neither compared nor shown: ``_validated_for`` = :func:`validation_key` of the
     ``(Sk, BLOCK_K)`` these lists have been checked against (set by the functions of this module, whose lists fit by
@@ -56,21 +60,32 @@ class MaskMetadata:
     schedule: Optional[torch.Tensor] = None
     schedule_mode: int = 0
     list_stats: Optional[Tuple[float, int]] = None
+    list_rotation: int = 0
     _validated_for: Optional[tuple] = field(default=None, repr=False, compare=False)
     _retiled: Optional[tuple] = field(default=None, repr=False, compare=False)
 
 
 def with_list_stats(md: "MaskMetadata") -> "MaskMetadata":
-    """Fills ``md.list_stats`` = (mean, longest) listed KV tiles per Q tile from the two count tensors (one host
-    synchronisation; the distinct planes of broadcast counts are read once) and returns ``md``."""
-    fl, pl = md.unmasked_lens, md.masked_lens
-    idx = tuple(slice(0, 1) if fl.stride(d) == 0 and pl.stride(d) == 0 else slice(None) for d in range(2))
-    total = (fl[idx].to(torch.int64) + pl[idx].to(torch.int64)).flatten()
+    """Fills ``md.list_stats`` = (mean, longest) listed KV tiles per Q tile from the two count tensors and
+    ``md.list_rotation`` (16 when the FULL lists slide along the keys from one Q tile to the next, as under a sliding
+    window; else 0) with one host synchronisation (the distinct planes of broadcast lists are read once); returns
+    ``md``."""
+    fl, pl, fid = md.unmasked_lens, md.masked_lens, md.unmasked_kv_ids
+    idx = tuple(slice(0, 1) if fl.stride(d) == 0 and pl.stride(d) == 0 and fid.stride(d) == 0 else slice(None)
+                for d in range(2))
+    fl_, pl_ = fl[idx].to(torch.int64), pl[idx].to(torch.int64)
+    total = (fl_ + pl_).flatten()
     if total.numel() == 0:
-        md.list_stats = (0.0, 0)
-    else:
-        both = torch.stack((total.sum(), total.max())).tolist()
-        md.list_stats = (both[0] / total.numel(), int(both[1]))
+        md.list_stats, md.list_rotation = (0.0, 0), 0
+        return md
+    # neighbouring Q tiles that both have FULL tiles, and those of them whose first FULL tile lies further on
+    first = fid[idx][..., 0]
+    both = (fl_[..., 1:] > 0) & (fl_[..., :-1] > 0)
+    slides = both & (first[..., 1:] > first[..., :-1])
+    got = torch.stack((total.sum(), total.max(), both.sum(), slides.sum(), fl_.sum())).tolist()
+    md.list_stats = (got[0] / total.numel(), int(got[1]))
+    # a sliding band: most neighbours slide, and the FULL lists are long enough for a rotation to matter
+    md.list_rotation = 16 if got[2] > 0 and got[3] > 0.5 * got[2] and got[4] / total.numel() >= 8 else 0
     return md
 
 

@@ -120,9 +120,9 @@ SHORT_LIST_KEYS = 512
 
 def _short_list_kernel(mask_metadata, dtype, D, BLOCK_Q, BLOCK_K, kernel) -> bool:
     """Whether this call runs the kernel for short lists (three workgroups per compute unit, 32 keys per step)."""
-    if kernel not in (None, "auto", "default", "short"):
-        raise ValueError(f"kernel must be 'auto', 'default' or 'short' (got {kernel!r})")
-    if kernel == "default":
+    if kernel not in (None, "auto", "default", "short", "rotated"):
+        raise ValueError(f"kernel must be 'auto', 'default', 'rotated' or 'short' (got {kernel!r})")
+    if kernel in ("default", "rotated"):
         return False
     has = (dtype in _DTYPES and D == 128 and BLOCK_Q == 128 and BLOCK_K >= 16 and BLOCK_K & (BLOCK_K - 1) == 0
            and getattr(mask_metadata, "packed_masks", None) is not None
@@ -157,7 +157,8 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
     few KV tiles (three workgroups per compute unit, 32 keys per step; bf16/fp16, D = 128, BLOCK_Q = 128, packed
     PARTIAL tiles, ``mask_metadata.list_stats`` with no list above 256 entries); None / "auto" = "short" when the
     metadata carries ``list_stats`` (``compute_mask_kernel(..., list_stats=True)``) that say the lists are short,
-    else "default".  The two agree within rounding.
+    else "default".  "rotated" = the default kernel with the FULL entries of Q tile qt walked from a start that depends
+    on qt (for sliding windows; "auto" takes it when ``mask_metadata.list_rotation`` says so).  All agree within rounding.
     """
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be [B,H,S,D]")
@@ -261,6 +262,14 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
             rc = lib.sa_sparse_attention_fwd_kernel(
                 *common, packed.data_ptr(), S(packed.stride()[:2]), lse.data_ptr() if return_lse else None,
                 S(lse.stride()) if return_lse else None, *tail[:-1], _native.SA_FWD_KERNEL_SHORT_LISTS, tail[-1])
+        elif (sched is None and q.dtype in _DTYPES
+              and (kernel == "rotated" or (kernel in (None, "auto") and getattr(mask_metadata, "list_rotation", 0) > 0))):
+            # the default kernel with the FULL entries of Q tile qt walked from a start that depends on qt
+            group = int(getattr(mask_metadata, "list_rotation", 0)) or 16
+            rc = lib.sa_sparse_attention_fwd_kernel(
+                *common, *((packed.data_ptr(), S(packed.stride()[:2])) if packed is not None else (None, None)),
+                lse.data_ptr() if return_lse else None, S(lse.stride()) if return_lse else None, *tail[:-1],
+                _native.SA_FWD_KERNEL_ROTATED | (group << 8), tail[-1])
         elif packed is not None or sched is not None or return_lse:
             pk = (packed.data_ptr(), S(packed.stride()[:2])) if packed is not None else (None, None)
             sc = ((sched.data_ptr(), sched.numel() * 4, int(getattr(mask_metadata, "schedule_mode", 0)))

@@ -1,6 +1,7 @@
-"""The forward's kernel for short lists (sa_sparse_attention_fwd_kernel with SA_FWD_KERNEL_SHORT_LISTS: three workgroups
-per compute unit, 32 keys per step) against the same checkers as the default kernel: the C oracle and fp32 masked SDPA
-(test_attn.py:40), max-abs <= 2e-2 on bf16/fp16 inputs; and against the default kernel within twice that."""
+"""The forward's other kernel forms (sa_sparse_attention_fwd_kernel): SA_FWD_KERNEL_SHORT_LISTS (three workgroups per
+compute unit, 32 keys per step) and SA_FWD_KERNEL_ROTATED_BY(G) (FULL entries walked from a start that depends on the
+Q tile), against the same checkers as the default kernel: the C oracle and fp32 masked SDPA (test_attn.py:40), max-abs
+<= 2e-2 on bf16/fp16 inputs; and against the default kernel within twice that."""
 import math
 
 import pytest
@@ -179,3 +180,64 @@ def test_lists_cut_at_the_cap_stay_inside_their_tensors(gpu):
     cut = mask.clone()
     cut[..., 256 * BK:] = False
     assert (o.float() - sdpa32(q, k, v, cut)).abs().max() <= TOL
+
+
+@pytest.mark.parametrize("BQ,BK,D", [(128, 32, 128), (128, 16, 128), (128, 64, 128), (128, 128, 64), (64, 32, 64), (256, 32, 128)])
+@pytest.mark.parametrize("group", [2, 8, 16, 64])
+def test_rotated_walk_of_the_full_entries(gpu, BQ, BK, D, group):
+    # a causal window (lists that slide), a prefix block and a dense stripe; bool mask and packed tiles; bf16
+    B, H, S = 1, 3, 2048
+    i = torch.arange(S, device=gpu)
+    mask = ((i[:, None] >= i[None, :]) & (i[:, None] - i[None, :] < 700)) | (i[None, :] < 200) | (i[:, None] >= 1800)
+    me = mask[None, None].expand(B, H, S, S)
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=group + BK, device=gpu)
+    want = sdpa32(q, k, v, mask)
+    for pack in (True, False):
+        md = compute_mask_kernel(me, BQ, BK, pack_partial=pack)
+        md.list_rotation = group
+        o, lse = sparse_attention(q, k, v, me, BQ, BK, md, return_lse=True)
+        torch.cuda.synchronize()
+        assert (o.float() - want).abs().max() <= TOL
+        assert torch.equal(o, sparse_attention(q, k, v, me, BQ, BK, md, kernel="rotated"))
+        o_def, lse_def = sparse_attention(q, k, v, me, BQ, BK, md, kernel="default", return_lse=True)
+        assert (o.float() - o_def.float()).abs().max() <= TOL and (lse - lse_def).abs().max() <= 6e-3
+    # the rotation permutes FULL entries only: a mask without FULL tiles gives the default kernel's bits
+    band = (i[:, None] - i[None, :]).abs() < 8
+    mdb = compute_mask_kernel(band[None, None].expand(B, H, S, S), BQ, BK)
+    assert int(mdb.unmasked_lens.sum()) == 0
+    ob = sparse_attention(q, k, v, band, BQ, BK, mdb, kernel="default")
+    mdb.list_rotation = group
+    assert torch.equal(ob, sparse_attention(q, k, v, band, BQ, BK, mdb))
+
+
+def test_rotation_hint_and_its_refusals(gpu):
+    S = 4096
+    i = torch.arange(S, device=gpu)
+    window = ((i[:, None] >= i[None, :]) & (i[:, None] - i[None, :] < 1024))[None, None]
+    assert compute_mask_kernel(window, 128, 32, list_stats=True).list_rotation == 16
+    assert compute_mask_kernel(W.composed_mask(4 * S, device=gpu)[None, None], 128, 32, list_stats=True).list_rotation == 16
+    assert compute_mask_kernel(W.causal_mask(S, gpu)[None, None], 128, 32, list_stats=True).list_rotation == 0
+    assert compute_mask_kernel(W.document_mask(S, seed=0, device=gpu, lo=200, hi=900)[None, None], 128, 32, list_stats=True).list_rotation == 0
+    assert compute_mask_kernel(W.random_block_mask(S, 128, 0.5, seed=1, device=gpu)[None, None], 128, 32, list_stats=True).list_rotation == 0
+    assert compute_mask_kernel(window, 128, 32).list_rotation == 0  # nothing is read back unless asked for
+    lib = _native.load()
+    st = _native.strides
+    B, H, D = 1, 1, 128
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=3, device=gpu)
+    md = compute_mask_kernel(window, 128, 32)
+    o = torch.empty_like(q)
+
+    def raw(kernel):
+        return lib.sa_sparse_attention_fwd_kernel(
+            q.data_ptr(), st(q.stride()), k.data_ptr(), st(k.stride()), v.data_ptr(), st(v.stride()), o.data_ptr(), st(o.stride()),
+            window.data_ptr(), st(window.stride()), md.unmasked_kv_ids.data_ptr(), st(md.unmasked_kv_ids.stride()),
+            md.unmasked_lens.data_ptr(), st(md.unmasked_lens.stride()), md.masked_kv_ids.data_ptr(), st(md.masked_kv_ids.stride()),
+            md.masked_lens.data_ptr(), st(md.masked_lens.stride()), None, None, None, None, B, H, S, S, D, 128, 32, 0,
+            D ** -0.5 / math.log(2), kernel, torch.cuda.current_stream().cuda_stream)
+
+    for bad in (_native.SA_FWD_KERNEL_ROTATED, _native.SA_FWD_KERNEL_ROTATED | (3 << 8), _native.SA_FWD_KERNEL_ROTATED | (128 << 8),
+                _native.SA_FWD_KERNEL_DEFAULT | (8 << 8)):
+        assert raw(bad) == _native.SA_ERR_INVALID_ARGUMENT
+    assert raw(_native.SA_FWD_KERNEL_ROTATED | (8 << 8)) == 0
+    torch.cuda.synchronize()
+    assert (o.float() - sdpa32(q, k, v, window[0, 0])).abs().max() <= TOL
