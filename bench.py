@@ -43,39 +43,67 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak, TFLOP/s
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E peak, GB/s
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this script and scaled by
-# the readings of a 1 GiB device copy in the same run (--calibrate-copy: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000
-# KiB).  The summaries with the commands are the files of TRAFFIC_SOURCE.
-TRAFFIC_FWD_CAUSAL_BYTES = 1.1748e9      # 864.3 MiB read + 256.0 MiB written (804 - 864 MiB read from box to box)
-TRAFFIC_CLASSIFY_1GIB_BYTES = 1.0744e9   # 1,048,628 + 327 KiB read, 256 + 45.5 KiB written
-# decode workloads, both kernels
-TRAFFIC_DECODE_BYTES = (4.2963e9, 1.6227e9)
-# backward of the headline workload, three passes + prepare: 4253.6 MiB read + 776 MiB written (4168 - 4311 MiB read)
-TRAFFIC_BWD_CAUSAL_BYTES = 5.274e9
-
-# where the constants above come from
-TRAFFIC_SOURCE = {
-    "forward": "profiles/sparse_fwd_kernel_causal_B8H32S4096D128.txt section 2",
-    "mask_classify": "profiles/mask_classify_kernels_mask_32768x32768.txt section 2",
-    "decode": "profiles/sparse_decode_kernel_B8H32Sk32768D128.txt",
-    "backward": "profiles/sparse_bwd_kernel_causal_B8H32S4096D128.txt",
+# HBM bytes per launch (read, written) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over
+# `bench.py --traffic-probe` and scaled by what the same counters read for the 1 GiB device copy of the same run
+# (`bench.py --traffic-summary` does the arithmetic).  profiles/hbm_traffic_all_kernels.txt holds the commands.
+TRAFFIC_BYTES = {
 }
-# The counters were read with the kernels built from sources of this digest (kernel_sources_sha16 below); the line
-# carries both digests, so a reader sees whether the traffic figures belong to the kernels that were timed.
-TRAFFIC_KERNEL_SOURCES_SHA16 = "f33b103d9f0f16d7"
+TRAFFIC_SOURCE = "profiles/hbm_traffic_all_kernels.txt"
+# The sources each kernel is built from.  The counters were read with kernels built from sources of the digests in
+# TRAFFIC_KERNEL_SOURCES_SHA16; the line carries those beside the digests of the sources in the tree, per kernel, so a
+# reader sees whether a traffic figure belongs to the kernel that was timed.
+KERNEL_FILES = {
+    "forward": ("sparse_fwd_kernel.h", "sparse_fwd_c32.hip", "fwd_common.h", "kernels.h", "sparse_fwd.hip", "sparse_fwd_inst.hip"),
+    "mask_classify": ("mask_classify.hip", "kernels.h"),
+    "decode": ("sparse_decode.hip", "fwd_common.h", "kernels.h"),
+    "backward": ("sparse_bwd.hip", "fwd_common.h", "kernels.h"),
+}
+TRAFFIC_KERNEL_SOURCES_SHA16 = {"forward": "", "mask_classify": "", "decode": "", "backward": ""}
 
 
-def kernel_sources_sha16():
-    """First 16 hex digits of the SHA-256 over the kernel sources (names and contents, in name order)."""
+def kernel_sources_sha16(which=None):
+    """First 16 hex digits of the SHA-256 over kernel sources (names and contents, in name order): the files of
+    KERNEL_FILES[which], or every file under csrc/ when `which` is None."""
     import glob
     import hashlib
 
+    files = sorted(glob.glob(os.path.join(ROOT, "sparseattention_amd", "csrc", "*")))
+    if which is not None:
+        files = [f for f in files if os.path.basename(f) in KERNEL_FILES[which]]
     h = hashlib.sha256()
-    for f in sorted(glob.glob(os.path.join(ROOT, "sparseattention_amd", "csrc", "*"))):
+    for f in files:
         h.update(os.path.basename(f).encode())
         with open(f, "rb") as fh:
             h.update(fh.read())
     return h.hexdigest()[:16]
+
+
+def traffic_of(workload, which):
+    """The traffic entries of a roofline object: read + written bytes per launch (None when never measured)."""
+    rw = TRAFFIC_BYTES.get(workload)
+    return {"traffic": (rw[0] + rw[1]) if rw else None, "traffic_read_written": list(rw) if rw else None,
+            "traffic_source": TRAFFIC_SOURCE if rw else None,
+            "traffic_kernel_sources_sha16": TRAFFIC_KERNEL_SOURCES_SHA16[which],
+            "kernel_sources_sha16": kernel_sources_sha16(which)}
+
+
+def forward_roofline(executed_flop, hbm_bytes, kernel_ms, workload, kernel):
+    """The forward against both of its floors: executed-tile flop at the bf16 MFMA peak, and q, k, v, o once through
+    HBM.  `bound` is the larger floor; achieved / peak / frac are quoted against it, both fractions side by side."""
+    t = kernel_ms * 1e-3
+    mfma_floor, hbm_floor = executed_flop / (PEAK_BF16_TFLOPS * 1e12), hbm_bytes / (PEAK_HBM_GBS * 1e9)
+    tf, gbs = executed_flop / t / 1e12, hbm_bytes / t / 1e9
+    out = {"bound": "mfma" if mfma_floor >= hbm_floor else "hbm"}
+    if out["bound"] == "mfma":
+        out.update({"achieved": round(tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4)})
+    else:
+        out.update({"achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)})
+    out.update({"mfma_frac": round(tf / PEAK_BF16_TFLOPS, 4), "hbm_frac": round(gbs / PEAK_HBM_GBS, 4),
+                "mfma_floor_ms": round(mfma_floor * 1e3, 4), "hbm_floor_ms": round(hbm_floor * 1e3, 4),
+                "flop_per_launch": executed_flop, "hbm_bytes_algorithmic": hbm_bytes, "kernel": kernel,
+                "kernel_ms": kernel_ms})
+    out.update(traffic_of(workload, "forward"))
+    return out
 
 
 SETTLE_LAUNCHES = 30
@@ -104,6 +132,13 @@ def parse():
                          "socket power, power cap, engine clock and temperatures from the amdgpu hwmon / sysfs files; "
                          "prints one JSON line with the figures per workload")
     ap.add_argument("--power-sampler", default=None, metavar="FILE", help=argparse.SUPPRESS)
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="instead of the benchmark: launch every timed workload of this script three times between "
+                         "marker kernels (for a rocprofv3 --pmc FETCH_SIZE or WRITE_SIZE run over this command), then a "
+                         "1 GiB device copy to scale the counters by; prints the workload names in order")
+    ap.add_argument("--traffic-summary", nargs=2, default=None, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="instead of the benchmark: read the two counter_collection.csv files of such runs and print "
+                         "HBM bytes read and written per launch of every workload (no GPU needed)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy a few times, so that a counter run over this command "
                          "holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -158,7 +193,11 @@ def forward_case(name, mask2d, q, k, v, steps, warmup, schedule=None, pack_parti
     B, H, S, D = q.shape
     BQ = block_q
     me = mask2d[None, None].expand(B, H, S, S)
-    md = compute_mask_kernel(me, BQ, block_k, pack_partial=pack_partial, schedule=schedule)
+    md = compute_mask_kernel(me, BQ, block_k, pack_partial=pack_partial, schedule=schedule, list_stats=True)
+    from sparseattention_amd.sparse_attn_kernel import _short_list_kernel
+    kernel = ("sparse_fwd_c32_kernel" if _short_list_kernel(md, q.dtype, D, BQ, block_k, None)
+              else "sparse_fwd_kernel" + (" (FULL entries walked from a start that depends on the Q tile)"
+                                          if md.list_rotation and schedule is None else ""))
     tiles_plane = int(md.unmasked_lens[0, 0].sum()) + int(md.masked_lens[0, 0].sum())
     partial_plane = int(md.masked_lens[0, 0].sum())
     # mean of the mask in row slabs (a [32768,32768] float copy would take 4 GiB)
@@ -175,8 +214,11 @@ def forward_case(name, mask2d, q, k, v, steps, warmup, schedule=None, pack_parti
         "kernel_ms": round(ev_ms, 4),
         "effective_tflops": round(useful / (wall_ms * 1e-3) / 1e12, 2),
         "executed_tflops": round(executed / (ev_ms * 1e-3) / 1e12, 2),
+        "list_entries_mean_longest": [round(md.list_stats[0], 2), md.list_stats[1]],
         "_executed_flop": executed,
         "_useful_flop": useful,
+        "_hbm_bytes": 2 * q.numel() * 2 + 2 * k.numel() * 2,  # q read, o written, k and v read once
+        "_kernel": kernel,
     }
 
 
@@ -222,7 +264,7 @@ def classify_case(steps, warmup):
         "pack_partial_ms": round(pack_ms, 4),
         "roofline": {"bound": "hbm", "achieved": round(nbytes / (ev_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(nbytes / (ev_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-                     "traffic": TRAFFIC_CLASSIFY_1GIB_BYTES, "traffic_source": TRAFFIC_SOURCE["mask_classify"],
+                     **traffic_of("mask_classify, composed mask 1 GiB", "mask_classify"),
                      "algorithmic_bytes": nbytes},
     }
 
@@ -284,8 +326,7 @@ def backward_case(q, k, v, steps, warmup):
         "ms": round(wall_ms, 4), "kernel_ms": round(ev_ms, 4),
         "executed_tflops": round(executed / (ev_ms * 1e-3) / 1e12, 1),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BWD_CAUSAL_BYTES,
-                     "traffic_source": TRAFFIC_SOURCE["backward"],
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), **traffic_of("backward, causal", "backward"),
                      "kernel": "sparse_bwd_kernel x3 (+ bwd_prepare_kernel)", "flop_per_launch": algorithmic},
     }
 
@@ -304,13 +345,7 @@ def decode_case(steps, warmup):
         if k is None:
             k, v = k2, v2
         del k2, v2
-        if Sq == 1:
-            mask = torch.ones(Sq, Sk, dtype=torch.bool, device="cuda")
-        else:
-            pos_q = torch.arange(Sk - Sq, Sk, device="cuda")[:, None]
-            pos_k = torch.arange(Sk, device="cuda")[None, :]
-            far = (torch.rand(Sk // BKd, generator=torch.Generator().manual_seed(2)) < 0.25).to("cuda").repeat_interleave(BKd)
-            mask = (pos_k <= pos_q) & ((pos_q - pos_k < 4096) | (pos_k < 512) | far[None, :])
+        mask = decode_mask(Sq, Sk, BKd)
         me = mask.expand(B, H, Sq, Sk)
         md = compute_mask_kernel(me, Sq, BKd)
         tiles = int(md.unmasked_lens.sum()) + int(md.masked_lens.sum())
@@ -322,7 +357,7 @@ def decode_case(steps, warmup):
             "ms": round(wall_ms, 4), "kernel_ms": round(ev_ms, 4),
             "roofline": {"bound": "hbm", "achieved": round(nbytes / (ev_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
                          "unit": "GB/s", "frac": round(nbytes / (ev_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-                         "traffic": TRAFFIC_DECODE_BYTES[case], "traffic_source": TRAFFIC_SOURCE["decode"],
+                         **traffic_of("decode, %d" % Sq, "decode"),
                          "algorithmic_bytes": nbytes,
                          "kernel": "sparse_decode_kernel (+ decode_merge_kernel)"},
         })
@@ -344,16 +379,15 @@ def long_configs(steps, warmup):
         q, k, v = W.qkv(Bc, Hc, Sc, D, torch.bfloat16, seed=0, device="cuda")
         mask = make()
         r = forward_case(name, mask, q, k, v, steps, warmup)
-        achieved = r["_executed_flop"] / (r["kernel_ms"] * 1e-3) / 1e12
         rows.append({
             "workload": name + "; tiles BLOCK_Q=128 BLOCK_K=32",
             "fraction_unmasked": r["fraction_unmasked"], "executed_tile_fraction": r["executed_tile_fraction"],
             "executed_tiles_per_plane": int(r["_executed_flop"] // (Bc * Hc * FLOP_PER_TILE)),
             "partial_tiles_per_plane": r["partial_tiles_per_plane"],
             "ms": r["ms"], "kernel_ms": r["kernel_ms"], "effective_tflops": r["effective_tflops"],
-            "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": "sparse_fwd_kernel",
-                         "flop_per_launch": r["_executed_flop"]},
+            "list_entries_mean_longest": r["list_entries_mean_longest"],
+            "roofline": forward_roofline(r["_executed_flop"], r["_hbm_bytes"], r["kernel_ms"],
+                                         "forward, " + name.split(":")[1].split(",")[0].strip(), r["_kernel"]),
         })
         del q, k, v, mask
         torch.cuda.empty_cache()
@@ -593,13 +627,146 @@ def power_trace(seconds):
     print(json.dumps(out))
 
 
+TRAFFIC_PROBE_LAUNCHES = 3
+MARKER_KERNEL = "validate_lists_kernel"  # (sa_validate_metadata: nothing else in a probe run launches it)
+
+
+def traffic_probe():
+    """Every workload this script times, TRAFFIC_PROBE_LAUNCHES launches each between two marker kernels (what runs
+    outside the markers - classification, warm-up - is not counted), the 1 GiB copy last."""
+    import torch
+    from sparseattention_amd import (_native, compute_backward_metadata, compute_mask_kernel, sparse_attention,
+                                     sparse_attention_backward, sparse_attention_decode, workloads as W)
+
+    lib = _native.load()
+    st = _native.strides
+    tiny = compute_mask_kernel(torch.ones(1, 1, 128, 128, dtype=torch.bool, device="cuda"), 128, 32, pack_partial=False)
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    names = []
+
+    def marker():
+        _native.check(lib.sa_validate_metadata(
+            tiny.unmasked_kv_ids.data_ptr(), st(tiny.unmasked_kv_ids.stride()), tiny.unmasked_lens.data_ptr(), st(tiny.unmasked_lens.stride()),
+            tiny.masked_kv_ids.data_ptr(), st(tiny.masked_kv_ids.stride()), tiny.masked_lens.data_ptr(), st(tiny.masked_lens.stride()),
+            1, 1, 128, 128, 128, 32, flag.data_ptr(), torch.cuda.current_stream().cuda_stream))
+
+    def measured(name, fn):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        marker()
+        for _ in range(TRAFFIC_PROBE_LAUNCHES):
+            fn()
+        marker()
+        torch.cuda.synchronize()
+        names.append(name)
+
+    def forward(name, mask2d, q, k, v):
+        Bc, Hc, Sc, _ = q.shape
+        me = mask2d[None, None].expand(Bc, Hc, Sc, Sc)
+        md = compute_mask_kernel(me, BQ, BK, list_stats=True)
+        measured("forward, " + name, lambda: sparse_attention(q, k, v, me, BQ, BK, mask_metadata=md))
+
+    q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=0, device="cuda")
+    forward("causal", W.causal_mask(S, "cuda"), q, k, v)
+    forward("dense", torch.ones(S, S, dtype=torch.bool, device="cuda"), q, k, v)
+    for p_ in (0.25, 0.5, 0.75, 0.9):
+        forward(f"p={p_}", W.random_block_mask(S, 128, p_, seed=int(p_ * 100), device="cuda"), q, k, v)
+    me = W.causal_mask(S, "cuda")[None, None].expand(B, H, S, S)
+    bmd = compute_backward_metadata(me)
+    o, lse = sparse_attention(q, k, v, me, BQ, BK, return_lse=True)
+    do = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(3)).to("cuda", torch.bfloat16)
+    measured("backward, causal", lambda: sparse_attention_backward(do, q, k, v, o, lse, me, bmd))
+    del q, k, v, o, lse, do, bmd, me
+    torch.cuda.empty_cache()
+    for name, Bc, Hc, Sc, make in (("documents", 4, 32, 16384, lambda: W.document_mask(16384, seed=0, device="cuda")),
+                                   ("composed", 1, 32, 32768, lambda: W.composed_mask(32768, device="cuda"))):
+        q, k, v = W.qkv(Bc, Hc, Sc, D, torch.bfloat16, seed=0, device="cuda")
+        forward(name, make(), q, k, v)
+        del q, k, v
+        torch.cuda.empty_cache()
+    big = W.composed_mask(32768, device="cuda")[None, None]
+    measured("mask_classify, composed mask 1 GiB", lambda: compute_mask_kernel(big, BQ, BK, pack_partial=False))
+    del big
+    torch.cuda.empty_cache()
+    Sk, BKd = 32768, 128
+    kd = vd = None
+    for Sq in (1, 16):
+        qd, k2, v2 = W.qkv(B, H, Sq, D, torch.bfloat16, seed=1, device="cuda", Sk=Sk)
+        if kd is None:
+            kd, vd = k2, v2
+        del k2, v2
+        mask = decode_mask(Sq, Sk, BKd)
+        med = mask.expand(B, H, Sq, Sk)
+        mdd = compute_mask_kernel(med, Sq, BKd)
+        measured("decode, %d" % Sq, lambda: sparse_attention_decode(qd, kd, vd, med, BKd, mask_metadata=mdd))
+    del kd, vd
+    torch.cuda.empty_cache()
+    src = torch.ones(1 << 28, dtype=torch.int32, device="cuda")  # 1 GiB read + 1 GiB written per copy
+    dst = torch.empty_like(src)
+    measured("copy 1 GiB", lambda: dst.copy_(src))
+    print(json.dumps({"traffic_probe_workloads": names, "launches_each": TRAFFIC_PROBE_LAUNCHES,
+                      "kernel_sources_sha16": {w: kernel_sources_sha16(w) for w in KERNEL_FILES}}))
+
+
+def traffic_summary(fetch_csv, write_csv):
+    """Per workload of a --traffic-probe run: counter units summed over the dispatches between an odd marker and the
+    next even one, per launch, scaled so that the copy of 1 GiB reads 2^30 bytes."""
+    import csv
+
+    names = ["forward, causal", "forward, dense", "forward, p=0.25", "forward, p=0.5", "forward, p=0.75", "forward, p=0.9",
+             "backward, causal", "forward, documents", "forward, composed", "mask_classify, composed mask 1 GiB",
+             "decode, 1", "decode, 16", "copy 1 GiB"]
+
+    def per_workload(path, counter):
+        rows = [r for r in csv.DictReader(open(path)) if r["Counter_Name"] == counter]
+        rows.sort(key=lambda r: int(r["Dispatch_Id"]))
+        sums, inside, acc = [], False, 0.0
+        for r in rows:
+            if MARKER_KERNEL in r["Kernel_Name"]:
+                if inside:
+                    sums.append(acc / TRAFFIC_PROBE_LAUNCHES)
+                inside, acc = not inside, 0.0
+            elif inside:
+                acc += float(r["Counter_Value"])
+        if len(sums) != len(names):
+            raise SystemExit(f"{path}: {len(sums)} marked spans, expected {len(names)}")
+        return sums
+
+    fetch, write = per_workload(fetch_csv, "FETCH_SIZE"), per_workload(write_csv, "WRITE_SIZE")
+    f_unit, w_unit = (1 << 30) / fetch[-1], (1 << 30) / write[-1]
+    out = {"bytes_per_FETCH_SIZE_unit": round(f_unit, 2), "bytes_per_WRITE_SIZE_unit": round(w_unit, 2), "workloads": {}}
+    for n, f, w in zip(names, fetch, write):
+        out["workloads"][n] = [round(f * f_unit), round(w * w_unit)]
+    print(json.dumps(out, indent=1))
+
+
+def decode_mask(Sq, Sk, BKd):
+    """The two decode workloads' masks: every key for one query row; else a causal window of 4096 keys, 512 sink keys
+    and a quarter of the far KV tiles."""
+    import torch
+
+    if Sq == 1:
+        return torch.ones(Sq, Sk, dtype=torch.bool, device="cuda")
+    pos_q = torch.arange(Sk - Sq, Sk, device="cuda")[:, None]
+    pos_k = torch.arange(Sk, device="cuda")[None, :]
+    far = (torch.rand(Sk // BKd, generator=torch.Generator().manual_seed(2)) < 0.25).to("cuda").repeat_interleave(BKd)
+    return (pos_k <= pos_q) & ((pos_q - pos_k < 4096) | (pos_k < 512) | far[None, :])
+
+
 def main():
     args = parse()
+    if args.traffic_summary:
+        traffic_summary(*args.traffic_summary)
+        return
     if args.power_sampler:
         power_sampler(args.power_sampler)
         return
     if args.power_trace > 0:
         power_trace(args.power_trace)
+        return
+    if args.traffic_probe:
+        traffic_probe()
         return
     if args.gpus != 1:
         print(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); the path has no multi-GPU leg.",
@@ -617,7 +784,6 @@ def main():
     q, k, v = W.qkv(B, H, S, D, torch.bfloat16, seed=0, device="cuda")
 
     head = forward_case("causal", W.causal_mask(S, "cuda"), q, k, v, args.steps, args.warmup)
-    achieved = head["_executed_flop"] / (head["kernel_ms"] * 1e-3) / 1e12
     result = {
         "metric": "effective TFLOP/s of the block-sparse forward (4*B*H*S*S*D*mean(mask)/time), B8 H32 S4096 D128 bf16",
         "value": head["effective_tflops"],
@@ -635,16 +801,12 @@ def main():
         "data": "synthetic",
         "config": {"workload": "configs[1]: causal bool mask [4096,4096] passed as a tensor, B=8 H=32 S=4096 D=128 bf16, "
                                "q/k/v ~ N(0,1), tiles BLOCK_Q=128 BLOCK_K=32, mask metadata precomputed "
-                               "(tile lists, bit-packed partial tiles; one workgroup per Q tile)",
+                               "(tile lists, bit-packed partial tiles, list statistics; one workgroup per Q tile)",
                    "executed_tiles_per_plane": int(head["_executed_flop"] // (B * H * FLOP_PER_TILE)),
-                   "partial_tiles_per_plane": head["partial_tiles_per_plane"]},
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_FWD_CAUSAL_BYTES,
-                     "traffic_source": TRAFFIC_SOURCE["forward"],
-                     "traffic_kernel_sources_sha16": TRAFFIC_KERNEL_SOURCES_SHA16,
-                     "kernel_sources_sha16": kernel_sources_sha16(),
-                     "kernel": "sparse_fwd_kernel", "kernel_ms": head["kernel_ms"],
-                     "flop_per_launch": head["_executed_flop"]},
+                   "partial_tiles_per_plane": head["partial_tiles_per_plane"],
+                   "list_entries_mean_longest": head["list_entries_mean_longest"]},
+        "roofline": forward_roofline(head["_executed_flop"], head["_hbm_bytes"], head["kernel_ms"], "forward, causal",
+                                     head["_kernel"]),
     }
     if not args.no_sweep:
         # (a launch after an idle gap runs up to 40 % slow and the next ten settle: never fewer than 10 warm-ups)
@@ -666,7 +828,11 @@ def main():
         for p in (0.25, 0.5, 0.75, 0.9):
             m = W.random_block_mask(S, 128, p, seed=int(p * 100), device="cuda")
             rows.append(forward_case(f"random blocks p={p}", m, q, k, v, sweep_steps, sweep_warm))
-        result["across_p"] = [{kk: vv for kk, vv in r.items() if not kk.startswith("_")} for r in rows]
+        result["across_p"] = [dict({kk: vv for kk, vv in r.items() if not kk.startswith("_")},
+                                   roofline=forward_roofline(r["_executed_flop"], r["_hbm_bytes"], r["kernel_ms"],
+                                                             "forward, " + r["mask"].replace(" (all True)", "").replace("random blocks ", ""),
+                                                             r["_kernel"]))
+                              for r in rows]
     if not args.no_classify:
         result["mask_classify"] = classify_case(max(10, args.steps // 2), max(3, args.warmup // 2))
         result["mask_terms"] = terms_case(max(10, args.steps // 2), max(3, args.warmup // 2))

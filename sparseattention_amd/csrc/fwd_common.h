@@ -99,6 +99,9 @@ constexpr float kNegInf = -__builtin_inff();
 // s_nop therefore stay INSIDE this asm statement: handing the address over as an "{m0}" input leaves the copy into
 // the (reserved) register to the compiler, with no guarantee of the wait state or that two loads do not share one
 // copy, and a build of that form ended in a GPU memory fault.
+// STREAM: the bytes are read once by the whole launch (the K/V rows of the few-rows kernels): the load carries the
+// non-temporal hint, with which a streaming read runs at 7.1 TB/s on this device against 6.3 TB/s without.
+template <bool STREAM = false>
 __device__ __forceinline__ void dma16(const void *base, uint32_t lane_offset, uint32_t lds_addr) {
     // the base is wave-uniform by construction; say so in a way the register allocator cannot miss
     const uint64_t b = (uint64_t)(uintptr_t)base;
@@ -106,13 +109,23 @@ __device__ __forceinline__ void dma16(const void *base, uint32_t lane_offset, ui
     const uint64_t ub = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b) |
                         ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32)) << 32);
     lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
-    asm volatile(
-        "s_mov_b32 m0, %2\n\t"
-        "s_nop 0\n\t"
-        "global_load_lds_dwordx4 %0, %1"
-        :
-        : "v"(lane_offset), "s"(ub), "s"(lds_addr)
-        : "memory");  // m0 is written; nothing else in these kernels keeps a value in it
+    if constexpr (STREAM) {
+        asm volatile(
+            "s_mov_b32 m0, %2\n\t"
+            "s_nop 0\n\t"
+            "global_load_lds_dwordx4 %0, %1 nt"
+            :
+            : "v"(lane_offset), "s"(ub), "s"(lds_addr)
+            : "memory");
+    } else {
+        asm volatile(
+            "s_mov_b32 m0, %2\n\t"
+            "s_nop 0\n\t"
+            "global_load_lds_dwordx4 %0, %1"
+            :
+            : "v"(lane_offset), "s"(ub), "s"(lds_addr)
+            : "memory");  // m0 is written; nothing else in these kernels keeps a value in it
+    }
 }
 
 // N dwords from N wave-uniform addresses by scalar loads that are issued back to back and share ONE wait.  Left to

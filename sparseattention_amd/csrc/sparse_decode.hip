@@ -151,7 +151,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64, 2) void sparse_decode_kernel(con
         for (int c = 0; c < NC; c++) kf[c] = *(const u32x4 *)(kp + 8 * c);
 #pragma unroll
         for (int i = 0; i < NLD; i++)
-            dma16(vbase + (int64_t)col * p.vs[2], ld_voff[i], vmine_lds + st * VBUF + RPI * i * ROWB);
+            dma16<true>(vbase + (int64_t)col * p.vs[2], ld_voff[i], vmine_lds + st * VBUF + RPI * i * ROWB);
         if ((t >> sh) >= F) {
 #pragma unroll
             for (int g = 0; g < 4; g++) {
