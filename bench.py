@@ -42,6 +42,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak, TFLOP/s
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E peak, GB/s
+PEAK_FP32_TFLOPS = 157.3   # MI355X dense fp32 MFMA peak, TFLOP/s
 
 # HBM bytes per launch (read, written) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over
 # `bench.py --traffic-probe` and scaled by what the same counters read for the 1 GiB device copy of the same run
@@ -362,6 +363,26 @@ def decode_case(steps, warmup):
                          "kernel": "sparse_decode_kernel (+ decode_merge_kernel)"},
         })
     return rows
+
+
+def fp32_case(steps, warmup):
+    """The headline workload with float32 q, k, v (the reference's kernel takes the element type of its inputs,
+    sparse_attn_kernel.py:98-101): v_mfma_f32_32x32x2_f32, nothing rounded below float32; against the fp32 MFMA peak."""
+    import torch
+    from sparseattention_amd import compute_mask_kernel, sparse_attention, workloads as W
+
+    q, k, v = W.qkv(B, H, S, D, torch.float32, seed=0, device="cuda")
+    me = W.causal_mask(S, "cuda")[None, None].expand(B, H, S, S)
+    md = compute_mask_kernel(me, BQ, BK)
+    tiles = int(md.unmasked_lens[0, 0].sum()) + int(md.masked_lens[0, 0].sum())
+    wall_ms, ev_ms = time_launches(lambda: sparse_attention(q, k, v, me, BQ, BK, mask_metadata=md), steps, warmup)
+    flop = tiles * B * H * FLOP_PER_TILE
+    tf = flop / (ev_ms * 1e-3) / 1e12
+    return {"workload": "configs[1] with float32 q, k, v, o (causal, B=8 H=32 S=4096 D=128, tiles 128x32, metadata precomputed)",
+            "ms": round(wall_ms, 4), "kernel_ms": round(ev_ms, 4),
+            "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(tf / PEAK_FP32_TFLOPS, 4), "traffic": None, "flop_per_launch": flop,
+                         "kernel": "sparse_fwd_f32_mfma_kernel", "dtype": "f32"}}
 
 
 def long_configs(steps, warmup):
@@ -841,6 +862,9 @@ def main():
         result["backward"] = backward_case(q, k, v, max(10, args.steps // 5), max(5, args.warmup // 2))
     del q, k, v
     torch.cuda.empty_cache()
+    if not args.no_sweep:
+        result["fp32_forward"] = fp32_case(max(5, args.steps // 10), max(3, args.warmup // 5))
+        torch.cuda.empty_cache()
     if not args.no_long:
         result["configs"] = long_configs(max(20, args.steps // 2), max(10, args.warmup))
     if not args.no_tiles:

@@ -24,6 +24,7 @@ UNITS = [("sparseattn_api.hip", "sparseattn_api.o", []), ("mask_classify.hip", "
          ("mask_terms.hip", "mask_terms.o", []),
          ("fwd_schedule.hip", "fwd_schedule.o", []), ("sparse_fwd.hip", "sparse_fwd.o", []),
          ("sparse_fwd_f32.hip", "sparse_fwd_f32.o", []), ("sparse_fwd_c32.hip", "sparse_fwd_c32.o", []),
+         ("sparse_fwd_f32_mfma.hip", "sparse_fwd_f32_mfma.o", []),
          ("sparse_decode.hip", "sparse_decode.o", []), ("sparse_bwd.hip", "sparse_bwd.o", [])]
 UNITS += [("sparse_fwd_inst.hip", f"sparse_fwd_dt{dt}_pk{pk}_ps{ps}.o",
            [f"-DSA_FWD_DT={dt}", f"-DSA_FWD_PK={pk}", f"-DSA_FWD_PS={ps}"])

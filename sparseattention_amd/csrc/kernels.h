@@ -139,6 +139,10 @@ hipError_t launch_fwd_c32(const FwdParams &p, int dtype, int D, int BQ, hipStrea
 // float32 q, k, v, o (the pointers of FwdParams then address floats; strides stay in elements): any BQ from 1 to 256
 // (to 128 at D = 256), any BK; reads the packed tiles when given, else the mask; no schedules.
 hipError_t launch_fwd_f32(const FwdParams &p, int D, int BQ, hipStream_t stream);
+// The same on the matrix unit (sparse_fwd_f32_mfma.hip) for the sizes it has (fwd_f32_mfma_has); launch_fwd_f32 takes
+// it whenever it can.
+bool fwd_f32_mfma_has(const FwdParams &p, int D, int BQ);
+hipError_t launch_fwd_f32_mfma(const FwdParams &p, int D, int BQ, hipStream_t stream);
 
 // Few query rows against a long K/V (decode): one Q tile of Sq <= 32 rows per (b, h), its list of KV tiles split
 // over `nsplit` workgroups whose partial results a second kernel merges.

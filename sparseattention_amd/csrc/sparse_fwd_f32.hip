@@ -171,6 +171,7 @@ hipError_t launch_d(const FwdParams &p, int BQ, hipStream_t stream) {
 
 hipError_t launch_fwd_f32(const FwdParams &p, int D, int BQ, hipStream_t stream) {
     if (BQ < 1 || BQ > (D > 128 ? 128 : 256)) return hipErrorInvalidValue;
+    if (fwd_f32_mfma_has(p, D, BQ)) return launch_fwd_f32_mfma(p, D, BQ, stream);
     switch (D) {
         case 64: return launch_d<64>(p, BQ, stream);
         case 128: return launch_d<128>(p, BQ, stream);

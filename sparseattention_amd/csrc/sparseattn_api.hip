@@ -349,7 +349,7 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
     fp.Sk = Sk;
     fp.nQ = Sq / BQ;
     fp.BK = BK;
-    fp.lbk = lbk;
+    fp.lbk = f32 ? (log2_exact(BK) > 0 ? log2_exact(BK) : 0) : lbk;  // (float32: any BLOCK_K; 0 unless a power of two)
     fp.mask_vec4 = (!use_packed && mask_strides[3] == 1 && aligned(mask, 4) && mask_strides[0] % 4 == 0 &&
                     mask_strides[1] % 4 == 0 && mask_strides[2] % 4 == 0)
                        ? 1

@@ -125,3 +125,32 @@ def test_tile_widths_that_are_no_power_of_two_and_the_widest_tile(gpu, D, BQ, BK
         assert (o.cpu() - want).abs().max() <= TOL32, f"packed={packed is not None}"
         ref = oracle.forward(q.numpy(), k.numpy(), v.numpy(), mask.numpy()[None, None], BQ, BK, p_round=0)
         assert np.abs(o.cpu().numpy() - ref).max() <= TOL32
+
+
+@pytest.mark.parametrize("D,BQ,BK", [(128, 128, 64), (128, 128, 128), (64, 32, 64), (64, 64, 256), (128, 64, 16), (64, 128, 16),
+                                     (128, 128, 32), (64, 32, 32)])
+def test_sizes_of_the_matrix_unit_kernel(gpu, D, BQ, BK):
+    # the float32 forward runs these sizes on v_mfma_f32_32x32x2_f32: every tile width class (16, 32, wider), every
+    # workgroup size, both mask sources, per-batch masks, a dead row, lists with FULL and PARTIAL entries, the lse
+    B, H, Sq, Sk = 2, 2, 512, 1024
+    g = torch.Generator().manual_seed(D + BQ + BK)
+    q = torch.randn(B, H, Sq, D, generator=g)
+    k = torch.randn(B, H, Sk, D, generator=g)
+    v = torch.randn(B, H, Sk, D, generator=g)
+    mask = torch.rand(B, 1, Sq, Sk, generator=g) < 0.3
+    mask[:, :, 9] = False
+    mask[:, :, 128:256, :512] = True
+    mask[:, :, 256:, 768:] = False
+    me = mask.expand(B, H, Sq, Sk)
+    want = sdpa_cpu(q, k, v, me)
+    s = torch.einsum("bhqd,bhkd->bhqk", q.double(), k.double()) / math.sqrt(D)
+    want_lse = torch.logsumexp(s.masked_fill(~me, float("-inf")), -1)
+    qg, kg, vg, mg = q.to(gpu), k.to(gpu), v.to(gpu), me.to(gpu)
+    for pack in (True, False):
+        md = compute_mask_kernel(mg, BQ, BK, pack_partial=pack)
+        o, lse = sparse_attention(qg, kg, vg, mg, BQ, BK, md, return_lse=True)
+        torch.cuda.synchronize()
+        assert (o.cpu() - want).abs().max() <= TOL32, f"pack={pack}"
+        assert torch.equal(o[:, :, 9].cpu(), torch.zeros(B, H, D))
+        live = ~torch.isneginf(want_lse)
+        assert torch.isneginf(lse.cpu()[~live]).all() and (lse.cpu().double()[live] - want_lse[live]).abs().max() <= 1e-5
