@@ -352,7 +352,7 @@ int sa_sparse_attention_fwd_kernel(const void *q, const int64_t q_strides[4], co
  *
  *   lists        output of sa_mask_classify for the same mask with BQ = Sq: shapes [B,H,1,Sk/BK] and [B,H,1]
  *                (stride entry 2 is ignored)
- *   BK           power of two >= 32
+ *   BK           power of two >= 16
  *   num_splits   workgroups per (b, h), 1..256, or 0 for sa_decode_num_splits(...)
  *   workspace    sa_decode_workspace_bytes(...) bytes of device memory, 16-byte aligned (may be NULL when that is 0,
  *                i.e. for one split); contents on return are unspecified
@@ -370,6 +370,24 @@ int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const 
                                const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int D, int BK,
                                int dtype, float sm_scale_log2, int num_splits, void *workspace, size_t workspace_bytes,
                                float *lse, const int64_t lse_strides[3], void *stream);
+
+/*
+ * sa_sparse_attention_decode with the bit-packed PARTIAL tiles (sa_mask_pack_partial with BQ = Sq for the same mask and
+ * lists; strides may be 0 on broadcast dimensions), or NULL.  When given, `mask` is not read and may be NULL, so the
+ * metadata that sa_mask_classify + sa_mask_pack_partial make for a mask serves the few-rows kernels as it serves the
+ * forward, and the bool tensor can be released.  At BK = 16 the packed rows are halfwords: Sq must then be even.
+ * Results are bit-identical to sa_sparse_attention_decode.
+ */
+int sa_sparse_attention_decode_ex(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                                  const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
+                                  const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
+                                  const int64_t full_ids_strides[4], const int32_t *full_lens,
+                                  const int64_t full_lens_strides[3], const int32_t *part_ids,
+                                  const int64_t part_ids_strides[4], const int32_t *part_lens,
+                                  const int64_t part_lens_strides[3], const uint8_t *packed,
+                                  const int64_t packed_strides[2], int B, int H, int Sq, int Sk, int D, int BK, int dtype,
+                                  float sm_scale_log2, int num_splits, void *workspace, size_t workspace_bytes, float *lse,
+                                  const int64_t lse_strides[3], void *stream);
 
 /*
  * Merge of n attention results over disjoint key ranges of the same queries (what sharding the key axis over

@@ -47,6 +47,7 @@ EXPORTS = (
     "sa_decode_num_splits",
     "sa_decode_workspace_bytes",
     "sa_sparse_attention_decode",
+    "sa_sparse_attention_decode_ex",
     "sa_merge_attention_parts",
     "sa_bwd_workspace_bytes",
     "sa_sparse_attention_bwd",
@@ -127,6 +128,11 @@ def load() -> ctypes.CDLL:
     )
     lib.sa_sparse_attention_decode.argtypes = (
         [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [ctypes.c_int] * 7 + [ctypes.c_float, ctypes.c_int]
+        + [_vp, ctypes.c_size_t] + [_vp, _i64p] + [_vp]
+    )
+    lib.sa_sparse_attention_decode_ex.restype = ctypes.c_int
+    lib.sa_sparse_attention_decode_ex.argtypes = (
+        [_vp, _i64p] * 4 + [_vp, _i64p] + [_vp, _i64p] * 4 + [_vp, _i64p] + [ctypes.c_int] * 7 + [ctypes.c_float, ctypes.c_int]
         + [_vp, ctypes.c_size_t] + [_vp, _i64p] + [_vp]
     )
     lib.sa_merge_attention_parts.restype = ctypes.c_int

@@ -155,8 +155,11 @@ struct DecodeParams {
     int64_t ms[4];                        // mask strides in bytes
     int64_t fis[3], fls[2], pis[3], pls[2];  // b, h (and entry) strides of the lists of the one Q tile
     int B, H, Sq, Sk;
-    int BK, lbk;    // KV tile width (a power of two >= 32) and its log2
+    int BK, lbk;    // KV tile width (a power of two >= 16) and its log2
     int mask_vec4;  // 1: mask columns are contiguous and 4-byte aligned
+    // Bit-packed PARTIAL tiles of the one Q tile (PackParams layout with BQ = Sq), or null: then the mask itself is read.
+    const uint8_t *packed;
+    int64_t pks[2];  // bytes between packed planes along b and h
     int nsplit;     // workgroups per (b, h)
     float *ws;      // [B*H][nsplit][Sq][D + 2] floats: unnormalised rows, then reference value and row sum
     float scale;    // softmax scale / ln 2

@@ -50,7 +50,10 @@ __device__ __forceinline__ void merge_parts(const float *part, int n, int64_t st
     }
 }
 
-template <int DT, int D>
+// PK: the mask entries of PARTIAL tiles come bit-packed from p.packed (sa_mask_pack_partial with BQ = Sq) instead of from
+// the bool mask.  B16: BLOCK_K = 16, two list entries per chunk of 32 keys (else BLOCK_K >= 32, BLOCK_K/32 chunks per
+// entry).
+template <int DT, int D, bool PK, bool B16>
 __global__ __launch_bounds__(kDecodeWaves * 64, 2) void sparse_decode_kernel(const DecodeParams p) {
     using E = Elem<DT>;
     constexpr int ROWB = D * 2;
@@ -76,8 +79,9 @@ __global__ __launch_bounds__(kDecodeWaves * 64, 2) void sparse_decode_kernel(con
     const int nKt = p.Sk >> p.lbk;
     const int F = min(max(p.full_lens[b * p.fls[0] + h * p.fls[1]], 0), nKt);
     const int NE = F + min(max(p.part_lens[b * p.pls[0] + h * p.pls[1]], 0), nKt - F);
-    const int sh = p.lbk - 5;  // chunks per list entry, log2
-    const int T = NE << sh;
+    constexpr int EPC = B16 ? 2 : 1;   // list entries per chunk
+    const int sh = B16 ? 0 : p.lbk - 5;  // chunks per list entry, log2
+    const int T = B16 ? (NE + 1) >> 1 : NE << sh;
     // this workgroup's chunks [t_lo, t_hi); this wave takes t_lo + wave, + 4, ...
     const int t_lo = (int)((unsigned)T * (unsigned)split / (unsigned)p.nsplit),
               t_hi = (int)((unsigned)T * (unsigned)(split + 1) / (unsigned)p.nsplit);  // T * nsplit < 2^31 (checked by the caller)
@@ -86,7 +90,10 @@ __global__ __launch_bounds__(kDecodeWaves * 64, 2) void sparse_decode_kernel(con
     // query row of this lane (rows past Sq are padding: zero queries, row 0's mask, never stored)
     const bool live = l32 < p.Sq;
     const int qrow = live ? l32 : 0;
-    const uint8_t *mrow = p.mask + b * p.ms[0] + h * p.ms[1] + (int64_t)qrow * p.ms[2];
+    const uint8_t *mrow = PK ? nullptr : p.mask + b * p.ms[0] + h * p.ms[1] + (int64_t)qrow * p.ms[2];
+    // this row's bits in the packed tile of a PARTIAL slot: BK/8 bytes per row, Sq rows per tile
+    const int64_t tile_bytes = (int64_t)p.Sq * (p.BK >> 3);
+    const uint8_t *prow = PK ? p.packed + b * p.pks[0] + h * p.pks[1] + (int64_t)qrow * (p.BK >> 3) : nullptr;
 
     // Q^T operand, scaled once: lane (l32, hh) keeps d = (D/2) hh + 8c .. +7 of its row for step c (K uses the same
     // order, so each lane's K bytes are contiguous)
@@ -135,50 +142,106 @@ __global__ __launch_bounds__(kDecodeWaves * 64, 2) void sparse_decode_kernel(con
     const uint32_t vmine_lds = lds0 + wave_u * 2 * VBUF;
     const int64_t koff_lane = (int64_t)l32 * p.ks[2] + (D / 2) * hh;
 
-    // list entry of chunk t -> first key column, PARTIAL or not
-    auto idx_load = [&](int t) -> int {
-        const int e = t >> sh;
-        const int idx = e < F ? fid[(int64_t)e * p.fis[2]] : pid[(int64_t)(e - F) * p.pis[2]];
-        return min(max(idx, 0), nKt - 1);
+    // list entries of chunk t (clamped into the row of tiles; an entry past the count reads as entry 0 and is masked out)
+    auto idx_load = [&](int t, int(&idx)[EPC]) {
+#pragma unroll
+        for (int j = 0; j < EPC; j++) {
+            const int e0 = B16 ? 2 * t + j : (t >> sh);
+            const int e = e0 < NE ? e0 : 0;
+            const int v = e < F ? fid[(int64_t)e * p.fis[2]] : pid[(int64_t)(e - F) * p.pis[2]];
+            idx[j] = min(max(v, 0), nKt - 1);
+        }
     };
-    auto col_of = [&](int t, int idx) -> int {
-        return (__builtin_amdgcn_readfirstlane(idx) << p.lbk) + ((t & ((1 << sh) - 1)) << 5);
+    // first key column of every entry of chunk t
+    auto cols_of = [&](int t, const int(&idx)[EPC], int(&col)[EPC]) {
+#pragma unroll
+        for (int j = 0; j < EPC; j++)
+            col[j] = (__builtin_amdgcn_readfirstlane(idx[j]) << p.lbk) + (B16 ? 0 : ((t & ((1 << sh) - 1)) << 5));
     };
-    // everything chunk t needs from memory: K into registers, V into LDS stage `st`, mask words if PARTIAL
-    auto issue = [&](int t, int col, int st, u32x4(&kf)[NC], uint32_t(&mk)[4]) {
-        const uint16_t *kp = kbase + (int64_t)col * p.ks[2] + koff_lane;
+    // what chunk t's entries are: bit j = entry j exists, bit 4 + j = it is PARTIAL
+    auto flags_of = [&](int t) -> unsigned {
+        unsigned f = 0u;
+#pragma unroll
+        for (int j = 0; j < EPC; j++) {
+            const int e = B16 ? 2 * t + j : (t >> sh);
+            if (e < NE) f |= (1u << j) | (e >= F ? (16u << j) : 0u);
+        }
+        return f;
+    };
+    constexpr unsigned ALL = (1u << EPC) - 1u;
+    constexpr int NMW = PK ? EPC : 4;  // mask words per lane and chunk
+    // everything chunk t needs from memory: K into registers, V into LDS stage `st`, mask words if it has a PARTIAL entry
+    auto issue = [&](int t, const int(&col)[EPC], int st, u32x4(&kf)[NC], uint32_t(&mk)[NMW]) {
+        const int kcol = B16 ? ((l32 < 16 ? col[0] : col[EPC - 1]) - (l32 & 16)) : col[0];  // (+ l32: this lane's key)
+        const uint16_t *kp = kbase + (int64_t)kcol * p.ks[2] + koff_lane;
 #pragma unroll
         for (int c = 0; c < NC; c++) kf[c] = *(const u32x4 *)(kp + 8 * c);
 #pragma unroll
-        for (int i = 0; i < NLD; i++)
-            dma16<true>(vbase + (int64_t)col * p.vs[2], ld_voff[i], vmine_lds + st * VBUF + RPI * i * ROWB);
-        if ((t >> sh) >= F) {
+        for (int i = 0; i < NLD; i++) {
+            // rows [RPI i, RPI i + RPI) of the chunk: with BLOCK_K = 16 the second half belongs to the second entry
+            const int vcol = B16 ? (RPI * i < 16 ? col[0] : col[EPC - 1] - 16) : col[0];
+            dma16<true>(vbase + (int64_t)vcol * p.vs[2], ld_voff[i], vmine_lds + st * VBUF + RPI * i * ROWB);
+        }
+        const unsigned fl = flags_of(t);
+        if (fl >> 4) {
+            if constexpr (PK) {
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int64_t cc = col + 8 * g + 4 * hh;
-                if (p.mask_vec4) {
-                    mk[g] = *(const uint32_t *)(mrow + cc);
-                } else {
-                    const uint8_t *m0 = mrow + cc * p.ms[3];
-                    mk[g] = (uint32_t)m0[0] | ((uint32_t)m0[p.ms[3]] << 8) | ((uint32_t)m0[2 * p.ms[3]] << 16) |
-                            ((uint32_t)m0[3 * p.ms[3]] << 24);
+                for (int j = 0; j < EPC; j++) {
+                    const int e = B16 ? 2 * t + j : (t >> sh);
+                    const uint8_t *a = prow + (int64_t)((fl >> (4 + j)) & 1u ? e - F : 0) * tile_bytes;
+                    if constexpr (B16) mk[j] = *(const uint16_t *)a;
+                    else mk[j] = *(const uint32_t *)(a + 4 * (t & ((1 << sh) - 1)));
+                }
+            } else {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int64_t cc = (B16 ? (g < 2 ? col[0] + 8 * g : col[EPC - 1] + 8 * (g - 2)) : col[0] + 8 * g) + 4 * hh;
+                    if (p.mask_vec4) {
+                        mk[g] = *(const uint32_t *)(mrow + cc);
+                    } else {
+                        const uint8_t *m0 = mrow + cc * p.ms[3];
+                        mk[g] = (uint32_t)m0[0] | ((uint32_t)m0[p.ms[3]] << 8) | ((uint32_t)m0[2 * p.ms[3]] << 16) |
+                                ((uint32_t)m0[3 * p.ms[3]] << 24);
+                    }
                 }
             }
         }
     };
     // one chunk: scores, mask, softmax update, O^T += V^T . P^T
-    auto compute = [&](int t, int st, const u32x4(&kf)[NC], const uint32_t(&mk)[4]) {
+    auto compute = [&](int t, int st, const u32x4(&kf)[NC], const uint32_t(&mk)[NMW]) {
         f32x16 s;
 #pragma unroll
         for (int i = 0; i < 16; i++) s[i] = 0.f;
 #pragma unroll
         for (int c = 0; c < NC; c++) s = E::mfma(kf[c], qf[c], s);
-        if ((t >> sh) >= F) {
+        const unsigned fl = flags_of(t);
+        if (fl != ALL) {  // a PARTIAL entry, or (BLOCK_K = 16) a second entry past the end of the list
+            if constexpr (PK) {
+                // bit k of w: key k of the chunk; FULL entries count as all ones, missing ones as zero
+                uint32_t w;
+                if constexpr (B16) {
+                    const uint32_t w0 = (fl & 16u) ? (mk[0] & 0xffffu) : ((fl & 1u) ? 0xffffu : 0u);
+                    const uint32_t w1 = (fl & 32u) ? (mk[EPC - 1] & 0xffffu) : ((fl & 2u) ? 0xffffu : 0u);
+                    w = w0 | (w1 << 16);
+                } else {
+                    w = (fl & 16u) ? mk[0] : ((fl & 1u) ? ~0u : 0u);
+                }
+                w >>= 4 * hh;  // this lane's keys are 8g + 4hh + jj
 #pragma unroll
-            for (int g = 0; g < 4; g++)
+                for (int g = 0; g < 4; g++)
 #pragma unroll
-                for (int jj = 0; jj < 4; jj++)
-                    if (((mk[g] >> (8 * jj)) & 0xffu) == 0u) s[4 * g + jj] = kNegInf;
+                    for (int jj = 0; jj < 4; jj++)
+                        if (((w >> (8 * g + jj)) & 1u) == 0u) s[4 * g + jj] = kNegInf;
+            } else {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int j = B16 ? (g >> 1) : 0;
+                    const uint32_t w = ((fl >> (4 + j)) & 1u) ? mk[g] : (((fl >> j) & 1u) ? 0x01010101u : 0u);
+#pragma unroll
+                    for (int jj = 0; jj < 4; jj++)
+                        if (((w >> (8 * jj)) & 0xffu) == 0u) s[4 * g + jj] = kNegInf;
+                }
+            }
         }
         float mx = kNegInf;
 #pragma unroll
@@ -218,17 +281,19 @@ __global__ __launch_bounds__(kDecodeWaves * 64, 2) void sparse_decode_kernel(con
     // ---- this wave's chunk stream: chunk t computes while chunk t + 4 loads and the index of t + 8 is fetched ----
     {
         u32x4 kf[2][NC];
-        uint32_t mk[2][4];
+        uint32_t mk[2][NMW];
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
-            for (int g = 0; g < 4; g++) mk[j][g] = 0u;
+            for (int g = 0; g < NMW; g++) mk[j][g] = 0u;
         int t = t_lo + wave_u;
-        int idxs[2] = {0, 0};  // idxs[s]: list index of the chunk that goes into stage s next
+        int idxs[2][EPC] = {};  // idxs[s]: list indices of the chunk that goes into stage s next
         if (t < t_hi) {
-            idxs[0] = idx_load(t);
-            if (t + kDecodeWaves < t_hi) idxs[1] = idx_load(t + kDecodeWaves);
-            issue(t, col_of(t, idxs[0]), 0, kf[0], mk[0]);
+            idx_load(t, idxs[0]);
+            if (t + kDecodeWaves < t_hi) idx_load(t + kDecodeWaves, idxs[1]);
+            int col[EPC];
+            cols_of(t, idxs[0], col);
+            issue(t, col, 0, kf[0], mk[0]);
         }
         for (; t < t_hi; t += 2 * kDecodeWaves) {
             static_for<2>([&](auto jc) {
@@ -241,12 +306,14 @@ __global__ __launch_bounds__(kDecodeWaves * 64, 2) void sparse_decode_kernel(con
 #pragma unroll
                 for (int c = 0; c < NC; c++) asm volatile("" ::"v"(kf[j][c]));
 #pragma unroll
-                for (int g = 0; g < 4; g++) asm volatile("" ::"v"(mk[j][g]));
-                asm volatile("" ::"v"(idxs[j ^ 1]));
+                for (int g = 0; g < NMW; g++) asm volatile("" ::"v"(mk[j][g]));
+#pragma unroll
+                for (int e = 0; e < EPC; e++) asm volatile("" ::"v"(idxs[j ^ 1][e]));
                 const int tn = tt + kDecodeWaves;
                 if (tn < t_hi) {
-                    const int col_n = col_of(tn, idxs[j ^ 1]);
-                    if (tn + kDecodeWaves < t_hi) idxs[j] = idx_load(tn + kDecodeWaves);
+                    int col_n[EPC];
+                    cols_of(tn, idxs[j ^ 1], col_n);
+                    if (tn + kDecodeWaves < t_hi) idx_load(tn + kDecodeWaves, idxs[j]);
                     issue(tn, col_n, j ^ 1, kf[j ^ 1], mk[j ^ 1]);
                 }
                 compute(tt, j, kf[j], mk[j]);
@@ -366,10 +433,10 @@ __global__ __launch_bounds__(256) void merge_parts_kernel(const MergeParams p) {
         p.lse[b * p.lses[0] + h * p.lses[1] + (int64_t)q * p.lses[2]] = L > 0.f ? M + __logf(L) : kNegInf;
 }
 
-template <int DT, int D>
-hipError_t launch_decode_one(const DecodeParams &p, hipStream_t stream) {
+template <int DT, int D, bool PK, bool B16>
+hipError_t launch_decode_kind(const DecodeParams &p, hipStream_t stream) {
     constexpr int smem = decode_smem_bytes<D>();
-    auto kern = sparse_decode_kernel<DT, D>;
+    auto kern = sparse_decode_kernel<DT, D, PK, B16>;
     static unsigned long long attr_done = 0;  // devices on which this kernel may use `smem` bytes of LDS
     if (const hipError_t e0 = allow_dynamic_smem(kern, smem, attr_done); e0 != hipSuccess) return e0;
     hipLaunchKernelGGL(kern, dim3(p.nsplit, p.B * p.H), dim3(kDecodeWaves * 64), smem, stream, p);
@@ -377,6 +444,13 @@ hipError_t launch_decode_one(const DecodeParams &p, hipStream_t stream) {
     if (e != hipSuccess || p.nsplit == 1) return e;
     hipLaunchKernelGGL((decode_merge_kernel<DT, D>), dim3(p.B * p.H), dim3(256), 0, stream, p);
     return hipGetLastError();
+}
+
+template <int DT, int D>
+hipError_t launch_decode_one(const DecodeParams &p, hipStream_t stream) {
+    const bool pk = p.packed != nullptr, b16 = p.BK == 16;
+    if (pk) return b16 ? launch_decode_kind<DT, D, true, true>(p, stream) : launch_decode_kind<DT, D, true, false>(p, stream);
+    return b16 ? launch_decode_kind<DT, D, false, true>(p, stream) : launch_decode_kind<DT, D, false, false>(p, stream);
 }
 
 }  // namespace

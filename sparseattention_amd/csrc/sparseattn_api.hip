@@ -737,7 +737,7 @@ int sa_mask_classify_terms(const int32_t *terms, int n_terms, const int32_t *doc
 }
 
 int sa_decode_num_splits(int B, int H, int Sq, int Sk, int BK) {
-    if (B <= 0 || H <= 0 || Sq <= 0 || Sq > 32 || Sk <= 0 || BK < 32 || Sk % BK) return 0;
+    if (B <= 0 || H <= 0 || Sq <= 0 || Sq > 32 || Sk <= 0 || BK < 16 || Sk % BK) return 0;
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess) return 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
@@ -756,20 +756,26 @@ size_t sa_decode_workspace_bytes(int B, int H, int Sq, int D, int num_splits) {
     return (size_t)B * H * num_splits * Sq * (size_t)(D + 2) * sizeof(float);
 }
 
-int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
-                               const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
-                               const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
-                               const int64_t full_ids_strides[4], const int32_t *full_lens,
-                               const int64_t full_lens_strides[3], const int32_t *part_ids,
-                               const int64_t part_ids_strides[4], const int32_t *part_lens,
-                               const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int D, int BK,
-                               int dtype, float sm_scale_log2, int num_splits, void *workspace, size_t workspace_bytes,
-                               float *lse, const int64_t lse_strides[3], void *stream) {
+}  // extern "C"
+
+namespace {
+int decode_impl(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4], const void *v,
+                const int64_t v_strides[4], void *o, const int64_t o_strides[4], const uint8_t *mask,
+                const int64_t mask_strides[4], const int32_t *full_ids, const int64_t full_ids_strides[4],
+                const int32_t *full_lens, const int64_t full_lens_strides[3], const int32_t *part_ids,
+                const int64_t part_ids_strides[4], const int32_t *part_lens, const int64_t part_lens_strides[3],
+                const uint8_t *packed, const int64_t packed_strides[2], int B, int H, int Sq, int Sk, int D, int BK,
+                int dtype, float sm_scale_log2, int num_splits, void *workspace, size_t workspace_bytes, float *lse,
+                const int64_t lse_strides[3], void *stream) {
     g_error[0] = 0;
-    if (!q || !k || !v || !o || !q_strides || !k_strides || !v_strides || !o_strides || !mask || !mask_strides ||
+    if (!q || !k || !v || !o || !q_strides || !k_strides || !v_strides || !o_strides ||
         !full_ids || !full_ids_strides || !full_lens || !full_lens_strides || !part_ids || !part_ids_strides ||
         !part_lens || !part_lens_strides)
         return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_decode: null pointer argument");
+    if (packed ? !packed_strides : (!mask || !mask_strides))
+        return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_decode: null pointer argument (%s)", packed ? "packed_strides" : "mask");
+    if (packed && (!aligned(packed, 4) || (B > 1 && packed_strides[0] % 4) || (H > 1 && packed_strides[1] % 4)))
+        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_decode_ex: packed needs a 4-byte aligned base and plane strides");
     if (const int rc = check_tiling(B, H, Sq, Sk, Sq > 0 ? Sq : 1, BK)) return rc;
     if (Sq > 32) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_decode: Sq %d (supported: 1..32 query rows)", Sq);
     if (D != 64 && D != 128) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_decode: head dim %d (supported: 64, 128)", D);
@@ -778,7 +784,10 @@ int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const 
     if (dtype != SA_DTYPE_BF16 && dtype != SA_DTYPE_FP16)
         return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_decode: dtype code %d (supported: 0 = bf16, 1 = fp16)", dtype);
     const int lbk = log2_exact(BK);
-    if (lbk < 5) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_decode: BLOCK_K %d (supported: powers of two >= 32)", BK);
+    if (lbk < 4) return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_decode: BLOCK_K %d (supported: powers of two >= 16)", BK);
+    // (a packed tile is Sq * BLOCK_K / 8 bytes; the kernel reads its rows as dwords, at BLOCK_K = 16 as halfwords)
+    if (packed && BK == 16 && (Sq & 1))
+        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_decode_ex: packed tiles at BLOCK_K 16 need an even number of query rows (got %d)", Sq);
     const int64_t *st[4] = {q_strides, k_strides, v_strides, o_strides};
     const void *ptr[4] = {q, k, v, o};
     const char *name[4] = {"q", "k", "v", "o"};
@@ -806,7 +815,10 @@ int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const 
     dp.k = static_cast<const uint16_t *>(k);
     dp.v = static_cast<const uint16_t *>(v);
     dp.o = static_cast<uint16_t *>(o);
-    dp.mask = mask;
+    dp.mask = packed ? nullptr : mask;
+    dp.packed = packed;
+    dp.pks[0] = packed ? packed_strides[0] : 0;
+    dp.pks[1] = packed ? packed_strides[1] : 0;
     dp.full_ids = full_ids;
     dp.full_lens = full_lens;
     dp.part_ids = part_ids;
@@ -817,7 +829,7 @@ int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const 
         dp.vs[i] = v_strides[i];
         dp.os[i] = o_strides[i];
     }
-    for (int i = 0; i < 4; i++) dp.ms[i] = mask_strides[i];
+    for (int i = 0; i < 4; i++) dp.ms[i] = packed ? 0 : mask_strides[i];
     // the lists of the one Q tile: b and h strides, and the stride along the entries
     dp.fis[0] = full_ids_strides[0];
     dp.fis[1] = full_ids_strides[1];
@@ -835,8 +847,8 @@ int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const 
     dp.Sk = Sk;
     dp.BK = BK;
     dp.lbk = lbk;
-    dp.mask_vec4 = (mask_strides[3] == 1 && aligned(mask, 4) && mask_strides[0] % 4 == 0 && mask_strides[1] % 4 == 0 &&
-                    mask_strides[2] % 4 == 0)
+    dp.mask_vec4 = (!packed && mask_strides[3] == 1 && aligned(mask, 4) && mask_strides[0] % 4 == 0 &&
+                    mask_strides[1] % 4 == 0 && mask_strides[2] % 4 == 0)
                        ? 1
                        : 0;
     dp.nsplit = num_splits;
@@ -853,6 +865,40 @@ int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const 
     const hipError_t e = sa::launch_decode(dp, dtype, D, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(SA_ERR_HIP, "sa_sparse_attention_decode: launch failed: %s", hipGetErrorString(e));
     return SA_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int sa_sparse_attention_decode(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                               const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
+                               const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
+                               const int64_t full_ids_strides[4], const int32_t *full_lens,
+                               const int64_t full_lens_strides[3], const int32_t *part_ids,
+                               const int64_t part_ids_strides[4], const int32_t *part_lens,
+                               const int64_t part_lens_strides[3], int B, int H, int Sq, int Sk, int D, int BK,
+                               int dtype, float sm_scale_log2, int num_splits, void *workspace, size_t workspace_bytes,
+                               float *lse, const int64_t lse_strides[3], void *stream) {
+    return decode_impl(q, q_strides, k, k_strides, v, v_strides, o, o_strides, mask, mask_strides, full_ids,
+                       full_ids_strides, full_lens, full_lens_strides, part_ids, part_ids_strides, part_lens,
+                       part_lens_strides, nullptr, nullptr, B, H, Sq, Sk, D, BK, dtype, sm_scale_log2, num_splits, workspace,
+                       workspace_bytes, lse, lse_strides, stream);
+}
+
+int sa_sparse_attention_decode_ex(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                                  const void *v, const int64_t v_strides[4], void *o, const int64_t o_strides[4],
+                                  const uint8_t *mask, const int64_t mask_strides[4], const int32_t *full_ids,
+                                  const int64_t full_ids_strides[4], const int32_t *full_lens,
+                                  const int64_t full_lens_strides[3], const int32_t *part_ids,
+                                  const int64_t part_ids_strides[4], const int32_t *part_lens,
+                                  const int64_t part_lens_strides[3], const uint8_t *packed,
+                                  const int64_t packed_strides[2], int B, int H, int Sq, int Sk, int D, int BK, int dtype,
+                                  float sm_scale_log2, int num_splits, void *workspace, size_t workspace_bytes, float *lse,
+                                  const int64_t lse_strides[3], void *stream) {
+    return decode_impl(q, q_strides, k, k_strides, v, v_strides, o, o_strides, mask, mask_strides, full_ids,
+                       full_ids_strides, full_lens, full_lens_strides, part_ids, part_ids_strides, part_lens,
+                       part_lens_strides, packed, packed_strides, B, H, Sq, Sk, D, BK, dtype, sm_scale_log2, num_splits,
+                       workspace, workspace_bytes, lse, lse_strides, stream);
 }
 
 size_t sa_bwd_workspace_bytes(int B, int H, int Sq) {

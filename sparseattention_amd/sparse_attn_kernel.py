@@ -96,10 +96,10 @@ def kernel_tiles(Sq: int, Sk: int, D: int, BLOCK_Q: int, BLOCK_K: int):
     compiler accepts (sparse_attn_kernel.py:149-185); the result does not depend on them."""
     BLOCK_Q, BLOCK_K = int(BLOCK_Q), int(BLOCK_K)
     ok_k = BLOCK_K >= 16 and BLOCK_K & (BLOCK_K - 1) == 0 and Sk % BLOCK_K == 0
-    if Sq < 32:  # the few-rows kernels: one Q tile of all rows, KV tiles of 32 keys or more, head dims up to 128
+    if Sq < 32:  # the few-rows kernels: one Q tile of all rows, KV tiles of 16 keys or more, head dims up to 128
         if D > 128:
             return None
-        if ok_k and BLOCK_K >= 32:
+        if ok_k:
             return Sq, BLOCK_K
         return next(((Sq, bk) for bk in (32, 64) if Sk % bk == 0), None)
     ok_q = [b for b in _KERNEL_BLOCK_Q if Sq % b == 0 and (D <= 128 or b in (64, 128))]  # (D above 128 runs as 256)
@@ -211,11 +211,9 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
         BLOCK_Q, BLOCK_K = tiles
         mask_metadata = again[1]
 
-    if Sq == BLOCK_Q and Sq < 32 and BLOCK_K >= 32 and not f32:
-        # one Q tile of fewer rows than the forward kernels tile by: the split-KV kernels.  They read the bool mask and
-        # use neither packed tiles nor a schedule, so metadata that carries those (compute_mask_kernel's default) runs too.
-        if mask is None:
-            raise ValueError("sparse_attention with fewer than 32 query rows reads the mask tensor: pass `mask`")
+    if Sq == BLOCK_Q and Sq < 32 and BLOCK_K >= 16 and not f32:
+        # one Q tile of fewer rows than the forward kernels tile by: the split-KV kernels (they use no schedule, and take
+        # the packed tiles where the metadata carries them, so `mask` may be None there as it may for the forward)
         return sparse_attention_decode(q, k, v, mask, BLOCK_K, mask_metadata, return_lse=return_lse)
     sm_scale = D ** (-0.5) * 1 / math.log(2)  # exp2 replaces exp (sparse_attn_kernel.py:152)
 
@@ -309,7 +307,7 @@ def sparse_attention_tiled(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ti
     return out[:, :, qo:qo + Sq].contiguous()
 
 
-def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor, BLOCK_K,
+def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor | None, BLOCK_K,
                             mask_metadata: MaskMetadata | None = None, num_splits: int = 0, *,
                             return_lse: bool = False):
     """:func:`sparse_attention` for Sq <= 32 query rows (decode, speculative or chunked-prefill tails), BLOCK_Q = Sq.
@@ -317,8 +315,9 @@ def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, m
     The reference lists decode kernels as future work (README.md:65); the result is defined by its forward
     (sparse_attn_kernel.py:149-185) called with ``BLOCK_Q = Sq``.  Every (b, h) has one Q tile, so its list of KV
     tiles is cut into ``num_splits`` ranges (0: chosen from the shape and the device) that run in parallel and are
-    merged afterwards.  ``mask_metadata``: from ``compute_mask_kernel(mask, Sq, BLOCK_K)``.  ``return_lse``: as in
-    :func:`sparse_attention`.
+    merged afterwards.  ``mask_metadata``: from ``compute_mask_kernel(mask, Sq, BLOCK_K)``; when it carries
+    ``packed_masks`` (the default there) the kernels read those bits and ``mask`` may be None (at BLOCK_K = 16 with an odd
+    number of query rows the bool mask is read instead).  ``return_lse``: as in :func:`sparse_attention`.
     """
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be [B,H,S,D]")
@@ -332,8 +331,11 @@ def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, m
     if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
         raise TypeError(f"q, k, v must share dtype bfloat16 or float16 (got {q.dtype}, {k.dtype}, {v.dtype})")
     sm_scale = D ** (-0.5) * 1 / math.log(2)
-    mask = mask.expand(B, H, Sq, Sk)
+    if mask is not None:
+        mask = mask.expand(B, H, Sq, Sk)
     if mask_metadata is None:
+        if mask is None:
+            raise ValueError("sparse_attention_decode needs the mask or mask_metadata with packed_masks")
         mask_metadata = compute_mask_kernel(mask, Sq, BLOCK_K)
     fid, fl = mask_metadata.unmasked_kv_ids, mask_metadata.unmasked_lens
     pid, pl = mask_metadata.masked_kv_ids, mask_metadata.masked_lens
@@ -343,7 +345,20 @@ def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, m
         if tuple(t.shape) != shape or t.dtype != torch.int32 or t.device != q.device:
             raise ValueError(f"mask_metadata.{name}: expected int32 {shape} on {q.device}, got {t.dtype} {tuple(t.shape)} on {t.device}")
     _checked_metadata(mask_metadata, Sk, BLOCK_K)
-    assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
+    packed = getattr(mask_metadata, "packed_masks", None)
+    if packed is not None:
+        shape = (B, H, 1, nK, Sq * int(BLOCK_K) // 8)
+        if (tuple(packed.shape) != shape or packed.dtype != torch.uint8 or packed.device != q.device
+                or packed.stride()[2:] != (nK * shape[4], shape[4], 1)):
+            raise ValueError(f"mask_metadata.packed_masks: expected uint8 {shape} on {q.device} with contiguous tiles, got "
+                             f"{packed.dtype} {tuple(packed.shape)} strides {packed.stride()}")
+        if int(BLOCK_K) == 16 and Sq % 2:  # (halfword rows: the kernels want an even number of them)
+            packed = None
+    if packed is None:
+        if mask is None:
+            raise ValueError("sparse_attention_decode without a mask tensor needs mask_metadata with packed_masks "
+                             "(and an even number of query rows at BLOCK_K = 16)")
+        assert mask.dtype == torch.bool, "mask must be a torch.bool tensor"
     Dk = _kernel_head_dim(D, (64, 128))
     qc, kc, vc = (_kernel_ready(_pad_head_dim(t, Dk)) for t in (q, k, v))
     o = torch.empty_like(qc)
@@ -355,11 +370,13 @@ def sparse_attention_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, m
         ws_bytes = lib.sa_decode_workspace_bytes(B, H, Sq, Dk, int(num_splits))
         ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=q.device) if ws_bytes else None
         lse = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device) if return_lse else None
-        rc = lib.sa_sparse_attention_decode(
+        rc = lib.sa_sparse_attention_decode_ex(
             qc.data_ptr(), S(qc.stride()), kc.data_ptr(), S(kc.stride()), vc.data_ptr(), S(vc.stride()),
-            o.data_ptr(), S(o.stride()), mask.data_ptr(), S(mask.stride()),
+            o.data_ptr(), S(o.stride()), mask.data_ptr() if mask is not None else None,
+            S(mask.stride()) if mask is not None else None,
             fid.data_ptr(), S(fid.stride()), fl.data_ptr(), S(fl.stride()),
             pid.data_ptr(), S(pid.stride()), pl.data_ptr(), S(pl.stride()),
+            packed.data_ptr() if packed is not None else None, S(packed.stride()[:2]) if packed is not None else None,
             B, H, Sq, Sk, Dk, int(BLOCK_K), _DTYPES[q.dtype], sm_scale, int(num_splits),
             ws.data_ptr() if ws is not None else None, ws_bytes,
             lse.data_ptr() if lse is not None else None, S(lse.stride()) if lse is not None else None,

@@ -47,7 +47,7 @@ def tile_mask(shape, BK, seed, device, p_empty=0.4, p_partial=0.2, keep_first=Tr
 
 @pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("Sq", [1, 2, 5, 8, 16, 31, 32])
-@pytest.mark.parametrize("BK", [32, 64, 256])
+@pytest.mark.parametrize("BK", [16, 32, 64, 256])
 def test_rows_and_tiles_against_oracle_and_sdpa(gpu, D, Sq, BK):
     B, H, Sk = 2, 3, 2048
     q, k, v = W.qkv(B, H, Sq, D, torch.bfloat16, seed=Sq + BK + D, device=gpu, Sk=Sk)
@@ -156,7 +156,7 @@ def test_errors(gpu):
     q8 = q[:, :, :8].contiguous()
     m8 = mask[:8]
     with pytest.raises(_native.SparseAttnError):
-        sparse_attention_decode(q8, k, v, m8, 16)  # BLOCK_K below 32
+        sparse_attention_decode(q8, k, v, m8, 8)  # BLOCK_K below 16
     with pytest.raises(ValueError):
         sparse_attention_decode(q8, k, v, m8, 32, num_splits=300)
     # a workspace that is too small, through the raw ABI
@@ -200,3 +200,56 @@ def test_lse_output(gpu, splits):
     # the row sum adds up P as rounded to bf16 (8 significant bits) for the P.V product: a sum that one term
     # dominates is off by up to 2^-8 of itself
     assert (lse[live].double() - want[live]).abs().max() <= 6e-3
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("Sq", [1, 2, 6, 16, 31, 32])
+@pytest.mark.parametrize("BK", [16, 32, 128])
+def test_packed_tiles_give_the_bits_of_the_bool_mask(gpu, D, Sq, BK):
+    # the same call fed from the bit-packed PARTIAL tiles and from the bool mask: bit-identical; from the packed tiles no
+    # mask tensor is needed (at BLOCK_K = 16 with an odd number of rows the wrapper reads the bool mask)
+    B, H, Sk = 2, 2, 4096
+    q, k, v = W.qkv(B, H, Sq, D, torch.bfloat16, seed=Sq + BK, device=gpu, Sk=Sk)
+    mask = tile_mask((B, 1, Sq, Sk), BK, seed=Sq + 7 * BK, device=gpu, p_partial=0.4).expand(B, H, Sq, Sk)
+    md = compute_mask_kernel(mask, Sq, BK)
+    assert md.packed_masks is not None
+    md_bool = compute_mask_kernel(mask, Sq, BK, pack_partial=False)
+    for splits in (1, 5):
+        o_pack, lse_pack = sparse_attention_decode(q, k, v, mask, BK, md, num_splits=splits, return_lse=True)
+        o_bool, lse_bool = sparse_attention_decode(q, k, v, mask, BK, md_bool, num_splits=splits, return_lse=True)
+        assert torch.equal(o_pack, o_bool) and torch.equal(lse_pack, lse_bool)
+    assert (o_pack.float() - sdpa32(q, k, v, mask)).abs().max() <= TOL
+    if BK > 16 or Sq % 2 == 0:
+        # blind to the mask tensor: none at all, or one with the wrong content
+        assert torch.equal(sparse_attention_decode(q, k, v, None, BK, md, num_splits=5), o_pack)
+        assert torch.equal(sparse_attention_decode(q, k, v, torch.zeros_like(mask), BK, md, num_splits=5), o_pack)
+        if Sq < 32:  # (32 rows are a Q tile of the forward kernels)
+            assert torch.equal(sparse_attention(q, k, v, None, Sq, BK, md), sparse_attention_decode(q, k, v, None, BK, md))
+    else:
+        with pytest.raises(ValueError, match="packed_masks"):
+            sparse_attention_decode(q, k, v, None, BK, md)
+
+
+def test_packed_entry_point_refusals(gpu):
+    lib = _native.load()
+    st = _native.strides
+    B, H, Sq, Sk, D, BK = 1, 1, 3, 512, 64, 16
+    q, k, v = W.qkv(B, H, Sq, D, torch.bfloat16, seed=1, device=gpu, Sk=Sk)
+    mask = tile_mask((B, H, Sq, Sk), BK, seed=2, device=gpu)
+    md = compute_mask_kernel(mask, Sq, BK)
+    o = torch.empty_like(q)
+
+    def raw(mask_t, packed):
+        return lib.sa_sparse_attention_decode_ex(
+            q.data_ptr(), st(q.stride()), k.data_ptr(), st(k.stride()), v.data_ptr(), st(v.stride()), o.data_ptr(), st(o.stride()),
+            mask_t.data_ptr() if mask_t is not None else None, st(mask_t.stride()) if mask_t is not None else None,
+            md.unmasked_kv_ids.data_ptr(), st(md.unmasked_kv_ids.stride()), md.unmasked_lens.data_ptr(), st(md.unmasked_lens.stride()),
+            md.masked_kv_ids.data_ptr(), st(md.masked_kv_ids.stride()), md.masked_lens.data_ptr(), st(md.masked_lens.stride()),
+            packed.data_ptr() if packed is not None else None, st(packed.stride()[:2]) if packed is not None else None,
+            B, H, Sq, Sk, D, BK, 0, D ** -0.5 / math.log(2), 1, None, 0, None, None, torch.cuda.current_stream().cuda_stream)
+
+    assert raw(None, None) == _native.SA_ERR_INVALID_ARGUMENT          # neither mask nor packed tiles
+    assert raw(None, md.packed_masks) == _native.SA_ERR_UNSUPPORTED    # halfword rows, odd row count
+    assert raw(mask, None) == 0
+    torch.cuda.synchronize()
+    assert (o.float() - sdpa32(q, k, v, mask)).abs().max() <= TOL

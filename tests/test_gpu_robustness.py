@@ -281,8 +281,8 @@ def test_pack_skips_list_entries_that_do_not_fit(gpu):
 
 
 def test_decode_route_with_default_metadata(gpu):
-    # compute_mask_kernel packs PARTIAL tiles by default; sparse_attention with fewer than 32 query rows must still
-    # reach the split-KV kernels (which read the bool mask) with that metadata
+    # compute_mask_kernel packs PARTIAL tiles by default; sparse_attention with fewer than 32 query rows reaches the
+    # split-KV kernels with that metadata (they read the packed tiles) and with the reference's four tensors alone
     B, H, Sq, Sk, D, BK = 2, 2, 8, 1024, 64, 32
     q, k, v = W.qkv(B, H, Sq, D, torch.bfloat16, seed=13, device=gpu, Sk=Sk)
     mask = (torch.rand(Sq, Sk, generator=torch.Generator().manual_seed(14)) < 0.3).to(gpu)
@@ -295,8 +295,10 @@ def test_decode_route_with_default_metadata(gpu):
     assert (o.float() - sdpa32(q, k, v, mask)).abs().max() <= TOL
     md2 = compute_mask_kernel(me, Sq, BK, schedule=None, pack_partial=False)
     assert torch.equal(o, sparse_attention(q, k, v, me, Sq, BK, md2))
+    # with the packed tiles no mask tensor is needed; without them it is
+    assert torch.equal(o, sparse_attention(q, k, v, None, Sq, BK, md))
     with pytest.raises(ValueError, match="mask"):
-        sparse_attention(q, k, v, None, Sq, BK, md)
+        sparse_attention(q, k, v, None, Sq, BK, md2)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

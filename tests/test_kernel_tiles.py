@@ -17,7 +17,8 @@ from sparseattention_amd.sparse_attn_kernel import _kernel_head_dim, kernel_tile
     ((64, 4096, 256, 64, 32), (64, 32)),
     ((48, 4096, 128, 16, 32), None),           # no Q tile divides 48 rows: the wrapper pads the rows
     ((16, 4096, 128, 16, 64), (16, 64)),       # fewer than 32 rows: the few-rows kernels, one Q tile
-    ((16, 4096, 128, 8, 16), (16, 32)),
+    ((16, 4096, 128, 8, 16), (16, 16)),        # (tiles of 16 keys they have)
+    ((16, 4096, 128, 8, 8), (16, 32)),
     ((16, 4096, 192, 16, 64), None),           # which stop at head dim 128
 ])
 def test_kernel_tiles(args, want):
