@@ -48,6 +48,18 @@ PEAK_FP32_TFLOPS = 157.3   # MI355X dense fp32 MFMA peak, TFLOP/s
 # `bench.py --traffic-probe` and scaled by what the same counters read for the 1 GiB device copy of the same run
 # (`bench.py --traffic-summary` does the arithmetic).  profiles/hbm_traffic_all_kernels.txt holds the commands.
 TRAFFIC_BYTES = {
+    "forward, causal": (875656057, 268435456),
+    "forward, dense": (808019140, 268435456),
+    "forward, p=0.25": (1470669822, 268435456),
+    "forward, p=0.5": (3048472525, 268435456),
+    "forward, p=0.75": (3040397950, 268435456),
+    "forward, p=0.9": (1486869018, 268435456),
+    "backward, causal": (4409989626, 813695157),
+    "forward, documents": (1774692337, 536870912),
+    "forward, composed": (1691989682, 268435456),
+    "mask_classify, composed mask 1 GiB": (1074106360, 308736),
+    "decode, 1": (4295523956, 344064),
+    "decode, 16": (1617159792, 5308757),
 }
 TRAFFIC_SOURCE = "profiles/hbm_traffic_all_kernels.txt"
 # The sources each kernel is built from.  The counters were read with kernels built from sources of the digests in
@@ -59,7 +71,8 @@ KERNEL_FILES = {
     "decode": ("sparse_decode.hip", "fwd_common.h", "kernels.h"),
     "backward": ("sparse_bwd.hip", "fwd_common.h", "kernels.h"),
 }
-TRAFFIC_KERNEL_SOURCES_SHA16 = {"forward": "", "mask_classify": "", "decode": "", "backward": ""}
+TRAFFIC_KERNEL_SOURCES_SHA16 = {"forward": "5ef90d7cd860a819", "mask_classify": "c6c9e6a7fb4bcc86", "decode": "39f4c61483f9cbce",
+                                "backward": "e2145cd4846343f8"}
 
 
 def kernel_sources_sha16(which=None):
@@ -137,6 +150,9 @@ def parse():
                     help="instead of the benchmark: launch every timed workload of this script three times between "
                          "marker kernels (for a rocprofv3 --pmc FETCH_SIZE or WRITE_SIZE run over this command), then a "
                          "1 GiB device copy to scale the counters by; prints the workload names in order")
+    ap.add_argument("--counter-summary", default=None, metavar="CSV",
+                    help="instead of the benchmark: read the counter_collection.csv of a rocprofv3 --pmc run over "
+                         "`bench.py --traffic-probe` and print every counter in it per launch of every workload (no GPU needed)")
     ap.add_argument("--traffic-summary", nargs=2, default=None, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="instead of the benchmark: read the two counter_collection.csv files of such runs and print "
                          "HBM bytes read and written per launch of every workload (no GPU needed)")
@@ -730,14 +746,44 @@ def traffic_probe():
                       "kernel_sources_sha16": {w: kernel_sources_sha16(w) for w in KERNEL_FILES}}))
 
 
+PROBE_WORKLOADS = ["forward, causal", "forward, dense", "forward, p=0.25", "forward, p=0.5", "forward, p=0.75", "forward, p=0.9",
+                   "backward, causal", "forward, documents", "forward, composed", "mask_classify, composed mask 1 GiB",
+                   "decode, 1", "decode, 16", "copy 1 GiB"]
+
+
+def counter_summary(path):
+    """Every counter of a --pmc run over --traffic-probe, summed over the dispatches of a workload's marked span and
+    divided by its launches."""
+    import csv
+
+    rows = list(csv.DictReader(open(path)))
+    rows.sort(key=lambda r: int(r["Dispatch_Id"]))
+    counters = sorted({r["Counter_Name"] for r in rows})
+    out = {n: {} for n in PROBE_WORKLOADS}
+    for c in counters:
+        sums, inside, acc = [], False, 0.0
+        for r in rows:
+            if r["Counter_Name"] != c:
+                continue
+            if MARKER_KERNEL in r["Kernel_Name"]:
+                if inside:
+                    sums.append(acc / TRAFFIC_PROBE_LAUNCHES)
+                inside, acc = not inside, 0.0
+            elif inside:
+                acc += float(r["Counter_Value"])
+        if len(sums) != len(PROBE_WORKLOADS):
+            raise SystemExit(f"{path}: {len(sums)} marked spans of {c}, expected {len(PROBE_WORKLOADS)}")
+        for n, v in zip(PROBE_WORKLOADS, sums):
+            out[n][c] = v
+    print(json.dumps(out, indent=1))
+
+
 def traffic_summary(fetch_csv, write_csv):
     """Per workload of a --traffic-probe run: counter units summed over the dispatches between an odd marker and the
     next even one, per launch, scaled so that the copy of 1 GiB reads 2^30 bytes."""
     import csv
 
-    names = ["forward, causal", "forward, dense", "forward, p=0.25", "forward, p=0.5", "forward, p=0.75", "forward, p=0.9",
-             "backward, causal", "forward, documents", "forward, composed", "mask_classify, composed mask 1 GiB",
-             "decode, 1", "decode, 16", "copy 1 GiB"]
+    names = PROBE_WORKLOADS
 
     def per_workload(path, counter):
         rows = [r for r in csv.DictReader(open(path)) if r["Counter_Name"] == counter]
@@ -779,6 +825,9 @@ def main():
     args = parse()
     if args.traffic_summary:
         traffic_summary(*args.traffic_summary)
+        return
+    if args.counter_summary:
+        counter_summary(args.counter_summary)
         return
     if args.power_sampler:
         power_sampler(args.power_sampler)
