@@ -164,14 +164,14 @@ int sa_sparse_attention_fwd(const void *q, const int64_t q_strides[4], const voi
                             int dtype, float sm_scale_log2, void *stream);
 
 /*
- * Check of caller-supplied lists before they are handed to a forward, decode or backward call, on the device and
- * without a host synchronisation: the counterpart of the guard the reference puts on every K/V and mask load
+ * Check of caller-supplied lists before they are handed to a forward, decode or backward call or to
+ * sa_mask_pack_partial, on the device and without a host synchronisation: the counterpart of the guard the reference puts on every K/V and mask load
  * (kv_offset < SEQLEN_K, sparse_attn_kernel.py:35,39,60).  ORs into *flag (a device int32 the caller has set to 0):
  *   1  a count is negative, or full_len + part_len exceeds Sk/BK for some Q tile
  *   2  a FULL index inside its count is outside [0, Sk/BK)      4  the same for a PARTIAL index
- * The caller reads the flag when it likes (with the results, say).  The attention kernels do not depend on it: they
- * clamp counts to the row of tiles and skip (forward) or clamp (decode, backward) indices out of range, so lists that
- * fail this check give wrong numbers, never an access outside the tensors.
+ * The caller reads the flag when it likes (with the results, say).  The kernels do not depend on it: they clamp
+ * counts to the row of tiles and skip (forward, sa_mask_pack_partial) or clamp (decode, backward) indices out of range,
+ * so lists that fail this check give wrong numbers (or unwritten packed slots), never an access outside the tensors.
  */
 int sa_validate_metadata(const int32_t *full_ids, const int64_t full_ids_strides[4], const int32_t *full_lens,
                          const int64_t full_lens_strides[3], const int32_t *part_ids, const int64_t part_ids_strides[4],
