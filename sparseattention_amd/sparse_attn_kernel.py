@@ -9,7 +9,8 @@ from . import _native
 from .mask_utils import MaskMetadata, Tiling, compute_mask_kernel, compute_mask_terms, validation_key
 
 _DTYPES = {torch.bfloat16: _native.SA_DTYPE_BF16, torch.float16: _native.SA_DTYPE_FP16}
-# the forward also takes float32 (a plain kernel on the vector units, for checks against fp32 references)
+# the forward also takes float32 (kernels that compute in float32 throughout: on the fp32 matrix instruction at head
+# dims 64 and 128 with Q tiles of 64 or 128 rows, on the vector units otherwise)
 _FWD_DTYPES = {**_DTYPES, torch.float32: _native.SA_DTYPE_FP32}
 
 
@@ -143,7 +144,7 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
     """softmax(q kᵀ / sqrt(D) + (mask ? 0 : -inf)) v, skipping KV tiles the mask empties.
 
     Signature and meaning follow sparse_attn_kernel.py:149-185: ``q`` [B,H,Sq,D], ``k``/``v``
-    [B,H,Sk,D] (bf16 or fp16 on the tuned kernels; float32 on a plain kernel that computes in float32 throughout; on a
+    [B,H,Sk,D] (bf16, fp16, or float32 on kernels that compute in float32 throughout; on a
     ROCm GPU), ``mask`` bool broadcastable to [B,H,Sq,Sk] with
     True = attend, tile sizes ``BLOCK_Q`` x ``BLOCK_K``, and optionally the metadata from
     :func:`compute_mask_kernel` so that preprocessing is paid once for many calls.
@@ -255,6 +256,8 @@ def sparse_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
         tail = (B, H, Sq, Sk, Dk, int(BLOCK_Q), int(BLOCK_K), _FWD_DTYPES[q.dtype], sm_scale,
                 torch.cuda.current_stream(q.device).cuda_stream)
         sched = getattr(mask_metadata, "schedule", None)
+        if kernel == "rotated" and (sched is not None or q.dtype not in _DTYPES):
+            raise ValueError("kernel='rotated' needs bf16/fp16 and mask_metadata without a schedule")
         lse = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device) if return_lse else None
         if _short_list_kernel(mask_metadata, q.dtype, Dk, int(BLOCK_Q), int(BLOCK_K), kernel):
             rc = lib.sa_sparse_attention_fwd_kernel(

@@ -164,6 +164,15 @@ def test_layouts_strides_and_cross_attention(gpu):
     q2 = torch.randn(B, H, D, Sq, generator=g, device=gpu).to(torch.bfloat16).transpose(-1, -2)
     o2 = sparse_attention(q2, k, v, mask, 64, 64)
     assert (o2.float() - sdpa32(q2, k, v, mask)).abs().max() <= TOL
+    # one K/V head for all query heads, as a view with head stride 0: no copy is made, same bits as from copies
+    k1, v1 = k[:, :1].expand(B, H, Sk, D), v[:, :1].expand(B, H, Sk, D)
+    assert k1.stride(1) == 0
+    o3 = sparse_attention(q, k1, v1, mask, 64, 64)
+    assert torch.equal(o3, sparse_attention(q, k1.contiguous(), v1.contiguous(), mask, 64, 64))
+    assert (o3.float() - sdpa32(q, k1, v1, mask)).abs().max() <= TOL
+    qd = q[:, :, :8]
+    od = sparse_attention(qd, k1, v1, mask[:, :, :8], 8, 64)  # the few-rows kernels
+    assert (od.float() - sdpa32(qd, k1, v1, mask[:, :, :8])).abs().max() <= TOL
 
 
 def test_wrapper_errors(gpu):

@@ -241,3 +241,10 @@ def test_rotation_hint_and_its_refusals(gpu):
     assert raw(_native.SA_FWD_KERNEL_ROTATED | (8 << 8)) == 0
     torch.cuda.synchronize()
     assert (o.float() - sdpa32(q, k, v, window[0, 0])).abs().max() <= TOL
+    # the Python wrapper refuses the request where no kernel can honour it, as it does for "short"
+    with pytest.raises(ValueError, match="rotated"):
+        sparse_attention(q.float(), k.float(), v.float(), window, 128, 32, md, kernel="rotated")
+    with pytest.raises(ValueError, match="rotated"):
+        sparse_attention(q, k, v, window, 128, 32, compute_mask_kernel(window, 128, 32, schedule="pairs"), kernel="rotated")
+    with pytest.raises(ValueError, match="kernel must be"):
+        sparse_attention(q, k, v, window, 128, 32, md, kernel="fast")
