@@ -319,7 +319,8 @@ int sa_sparse_attention_fwd_lse(const void *q, const int64_t q_strides[4], const
  *   SA_FWD_KERNEL_ROTATED_BY(G)  the default kernel, with Q tile qt walking its FULL entries (all but the first chunk
  *                              of 64 keys) from a start BQ/64 * (G - 1 - qt mod G) chunks further on, wrapping
  *                              around; 2 <= G <= 64, a power of two (a Q tile whose FULL list is shorter than the
- *                              largest start halves G until it fits).  For banded masks (sliding windows): the windows of neighbouring Q tiles
+ *                              largest start halves G until it fits); bf16 or fp16 (else SA_ERR_UNSUPPORTED).
+ *                              For banded masks (sliding windows): the windows of neighbouring Q tiles
  *                              are BQ keys apart, so walked from the front they read the same K/V rows two chunks
  *                              apart and find them evicted from L2; walked this way G neighbours read them at the
  *                              same time.  The reference fixes FULL entries before PARTIAL ones

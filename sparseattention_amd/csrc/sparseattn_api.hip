@@ -265,9 +265,11 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
     if (D <= 0) return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd: D must be positive (got %d)", D);
     if (!(sm_scale_log2 > 0.f) || !(sm_scale_log2 < 3.0e38f))
         return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd: sm_scale_log2 must be positive and finite");
-    const bool f32 = dtype == SA_DTYPE_FP32;  // the plain float32 kernel: any BLOCK_Q up to 256, any BLOCK_K
+    const bool f32 = dtype == SA_DTYPE_FP32;  // the float32 kernels: any BLOCK_Q up to 256, any BLOCK_K
     if (dtype != SA_DTYPE_BF16 && dtype != SA_DTYPE_FP16 && !f32)
         return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: dtype code %d (supported: 0 = bf16, 1 = fp16, 2 = fp32)", dtype);
+    if (f32 && kernel == SA_FWD_KERNEL_ROTATED)
+        return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd_kernel: the rotated walk needs bf16 or fp16");
     if (D != 64 && D != 128 && D != 256)
         return fail(SA_ERR_UNSUPPORTED, "sa_sparse_attention_fwd: head dim %d (supported: 64, 128, 256)", D);
     int lbk = 0;
@@ -355,7 +357,7 @@ int forward_impl(const void *q, const int64_t q_strides[4], const void *k, const
                        ? 1
                        : 0;
     fp.scale = sm_scale_log2;
-    fp.rot = (kernel == SA_FWD_KERNEL_ROTATED && !f32) ? rot_group : 0;
+    fp.rot = kernel == SA_FWD_KERNEL_ROTATED ? rot_group : 0;
     fp.lse = nullptr;
     if (lse) {
         if (!lse_strides) return fail(SA_ERR_INVALID_ARGUMENT, "sa_sparse_attention_fwd_lse: null pointer argument (lse_strides)");

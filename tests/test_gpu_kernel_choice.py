@@ -227,12 +227,12 @@ def test_rotation_hint_and_its_refusals(gpu):
     md = compute_mask_kernel(window, 128, 32)
     o = torch.empty_like(q)
 
-    def raw(kernel):
+    def raw(kernel, dtype=0):
         return lib.sa_sparse_attention_fwd_kernel(
             q.data_ptr(), st(q.stride()), k.data_ptr(), st(k.stride()), v.data_ptr(), st(v.stride()), o.data_ptr(), st(o.stride()),
             window.data_ptr(), st(window.stride()), md.unmasked_kv_ids.data_ptr(), st(md.unmasked_kv_ids.stride()),
             md.unmasked_lens.data_ptr(), st(md.unmasked_lens.stride()), md.masked_kv_ids.data_ptr(), st(md.masked_kv_ids.stride()),
-            md.masked_lens.data_ptr(), st(md.masked_lens.stride()), None, None, None, None, B, H, S, S, D, 128, 32, 0,
+            md.masked_lens.data_ptr(), st(md.masked_lens.stride()), None, None, None, None, B, H, S, S, D, 128, 32, dtype,
             D ** -0.5 / math.log(2), kernel, torch.cuda.current_stream().cuda_stream)
 
     for bad in (_native.SA_FWD_KERNEL_ROTATED, _native.SA_FWD_KERNEL_ROTATED | (3 << 8), _native.SA_FWD_KERNEL_ROTATED | (128 << 8),
@@ -240,6 +240,7 @@ def test_rotation_hint_and_its_refusals(gpu):
         assert raw(bad) == _native.SA_ERR_INVALID_ARGUMENT
     assert raw(_native.SA_FWD_KERNEL_ROTATED | (8 << 8)) == 0
     torch.cuda.synchronize()
+    assert raw(_native.SA_FWD_KERNEL_ROTATED | (8 << 8), dtype=_native.SA_DTYPE_FP32) == _native.SA_ERR_UNSUPPORTED
     assert (o.float() - sdpa32(q, k, v, window[0, 0])).abs().max() <= TOL
     # the Python wrapper refuses the request where no kernel can honour it, as it does for "short"
     with pytest.raises(ValueError, match="rotated"):
