@@ -48,18 +48,18 @@ PEAK_FP32_TFLOPS = 157.3   # MI355X dense fp32 MFMA peak, TFLOP/s
 # `bench.py --traffic-probe` and scaled by what the same counters read for the 1 GiB device copy of the same run
 # (`bench.py --traffic-summary` does the arithmetic).  profiles/hbm_traffic_all_kernels.txt holds the commands.
 TRAFFIC_BYTES = {
-    "forward, causal": (875656057, 268435456),
-    "forward, dense": (808019140, 268435456),
-    "forward, p=0.25": (1470669822, 268435456),
-    "forward, p=0.5": (3048472525, 268435456),
-    "forward, p=0.75": (3040397950, 268435456),
-    "forward, p=0.9": (1486869018, 268435456),
-    "backward, causal": (4409989626, 813695157),
-    "forward, documents": (1774692337, 536870912),
-    "forward, composed": (1691989682, 268435456),
+    "forward, causal": (853480159, 268435456),
+    "forward, dense": (808017050, 268436693),
+    "forward, p=0.25": (1357508698, 268435456),
+    "forward, p=0.5": (2852257992, 268435456),
+    "forward, p=0.75": (2931904415, 268435456),
+    "forward, p=0.9": (1417653896, 268435456),
+    "backward, causal": (4305326450, 813694976),
+    "forward, documents": (1721826894, 536870912),
+    "forward, composed": (1612058763, 268435456),
     "mask_classify, composed mask 1 GiB": (1074106360, 308736),
-    "decode, 1": (4295523956, 344064),
-    "decode, 16": (1617159792, 5308757),
+    "decode, 1": (4295526174, 344064),
+    "decode, 16": (1617159835, 5308501),
 }
 TRAFFIC_SOURCE = "profiles/hbm_traffic_all_kernels.txt"
 # The sources each kernel is built from.  The counters were read with kernels built from sources of the digests in
@@ -71,8 +71,8 @@ KERNEL_FILES = {
     "decode": ("sparse_decode.hip", "fwd_common.h", "kernels.h"),
     "backward": ("sparse_bwd.hip", "fwd_common.h", "kernels.h"),
 }
-TRAFFIC_KERNEL_SOURCES_SHA16 = {"forward": "5ef90d7cd860a819", "mask_classify": "c6c9e6a7fb4bcc86", "decode": "39f4c61483f9cbce",
-                                "backward": "e2145cd4846343f8"}
+TRAFFIC_KERNEL_SOURCES_SHA16 = {"forward": "bc08ea58e0414ab6", "mask_classify": "c6c9e6a7fb4bcc86", "decode": "39f4c61483f9cbce",
+                                "backward": "44a7b516fda679c3"}
 
 
 def kernel_sources_sha16(which=None):

@@ -314,7 +314,8 @@ __global__ __launch_bounds__(256, 2) void sparse_bwd_kernel(const BwdParams p) {
     for (int i = 0; i < 32 * PPR_O / 64; i++) {
         const int idx = 64 * i + lane, r = idx / PPR_O, pc = idx % PPR_O;
         const u32x4 x = *(const u32x4 *)(ob + r * OROW + 16 * pc);
-        *(u32x4 *)(o0 + (int64_t)r * p.outs[2] + 8 * pc) = x;
+        // (written once, whole rows: a streaming store leaves the streamed operands' lines in L2 alone)
+        __builtin_nontemporal_store(x, (u32x4 *)(o0 + (int64_t)r * p.outs[2] + 8 * pc));
     }
 }
 
@@ -329,8 +330,9 @@ __global__ __launch_bounds__(256) void bwd_prepare_kernel(const BwdPrepParams p)
     const int q = (int)(row % p.Sq);
     const int bh = (int)(row / p.Sq);
     const int b = bh / p.H, h = bh - b * p.H;
-    const u32x4 a = *(const u32x4 *)(p.o + b * p.os[0] + h * p.os[1] + (int64_t)q * p.os[2] + 8 * part);
-    const u32x4 g = *(const u32x4 *)(p.d_o + b * p.dos[0] + h * p.dos[1] + (int64_t)q * p.dos[2] + 8 * part);
+    // (read once, whole rows: streaming loads, which this device serves faster than loads that keep their lines in L2)
+    const u32x4 a = __builtin_nontemporal_load((const u32x4 *)(p.o + b * p.os[0] + h * p.os[1] + (int64_t)q * p.os[2] + 8 * part));
+    const u32x4 g = __builtin_nontemporal_load((const u32x4 *)(p.d_o + b * p.dos[0] + h * p.dos[1] + (int64_t)q * p.dos[2] + 8 * part));
     float sum = 0.f;
 #pragma unroll
     for (int e = 0; e < 4; e++) {

@@ -493,7 +493,7 @@ __global__ __launch_bounds__(256, 3) void sparse_fwd_c32_kernel(const FwdParams 
         for (int i = 0; i < 8; i++) {
             const int idx = 64 * i + lane2, r = idx >> 4, pc = idx & 15;
             const u32x4 x = *(const u32x4 *)(ob + r * OROW + 16 * pc);
-            *(u32x4 *)(o0 + (int64_t)r * p.os[2] + 8 * pc) = x;
+            __builtin_nontemporal_store(x, (u32x4 *)(o0 + (int64_t)r * p.os[2] + 8 * pc));  // (streaming, as in sparse_fwd_kernel)
         }
     }
 }

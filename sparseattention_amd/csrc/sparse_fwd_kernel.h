@@ -785,7 +785,8 @@ __global__ __launch_bounds__(NW * 64, (NW >= 4 && D <= 128) ? 2 : 1) void sparse
         for (int i = 0; i < 32 * PPR / 64; i++) {
             const int idx = 64 * i + lane, r = idx / PPR, pc = idx % PPR;
             const u32x4 x = *(const u32x4 *)(ob + r * OROW + 16 * pc);
-            *(u32x4 *)(o0 + (int64_t)r * p.os[2] + 8 * pc) = x;
+            // (written once, whole rows: a streaming store leaves the lines of K and V in L2 alone)
+            __builtin_nontemporal_store(x, (u32x4 *)(o0 + (int64_t)r * p.os[2] + 8 * pc));
         }
     };
 
